@@ -1,0 +1,137 @@
+/*
+ * q8_0_abi.h -- C ABI of the MI355X (gfx950) Q8_0 mat-mul path.
+ *
+ * Plain C, no HIP or torch types: pointers, sizes, an opaque stream.  Every pointer is a DEVICE
+ * pointer unless the parameter name starts with host_.  `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream).  Calls are asynchronous on that stream and return once the work is
+ * enqueued; nothing here allocates or frees caller-visible memory except nh_malloc / nh_free.
+ * Return value: 0 on success, a negative nh_status for a rejected argument, or a positive
+ * hipError_t value when the HIP runtime reported one.  No exception crosses this boundary.
+ *
+ * What each entry point replaces in the reference (paths relative to include/nihilus-incl/):
+ * the reference has no FFI for this path; its boundary is the class-template specialisation point
+ * kernel_dispatcher_impl<config, core_traits, device, arch, ...>::impl (common/kernel_traits.hpp:382-383,
+ * called from infra/monolithic_dispatcher.hpp:41-63).  The C++ header mul_mat_dispatch.hpp supplies
+ * those specialisations for device_types::gpu and forwards to the functions below.
+ *
+ * Data layouts
+ *   "blocks"  the reference's wire layout: rows of packed 34-byte block_q8_0 { fp16 d; int8 qs[32] }
+ *             (common/data_types.hpp:38-44), row stride (K/32)*34 bytes, row-major.
+ *   "tiled"   this library's device layout for streaming and MFMA operands, same byte count per
+ *             block.  Rows are padded to a multiple of 32, K must be a multiple of 128.  The matrix
+ *             is a sequence of 4352-byte macro-tiles indexed [row strip s = r/32][k group g = k/128]:
+ *               bytes [t*1024 + 16*l + i], t<4, l<64, i<16 : quant (16*(l/32) + i) of block 4g+t of
+ *                                                          row 32s + (l%32)
+ *               bytes [4096 + 8*r + 2*t]                  : fp16 d of block 4g+t of row 32s + r
+ *             so one 64-lane wavefront fetches a 32-row x 32-quant tile with a single fully
+ *             coalesced 16-byte-per-lane load that already is a v_mfma_i32_32x32x32_i8 operand.
+ */
+#ifndef NIHILUS_AMD_Q8_0_ABI_H
+#define NIHILUS_AMD_Q8_0_ABI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NH_Q8_0_QK 32 /* Q_SIZE, common/data_types.hpp:28 */
+#define NH_Q8_0_BLOCK_BYTES 34 /* sizeof(block_q8_0<half>), common/data_types.hpp:44 */
+
+typedef enum nh_status {
+	NH_OK			   = 0,
+	NH_ERR_NULL_POINTER = -1, /* a required pointer is NULL */
+	NH_ERR_ALIGNMENT   = -2, /* a pointer is not 16-byte aligned (arena slices are 64-byte aligned, infra/core_traits.hpp:130) */
+	NH_ERR_SHAPE	   = -3, /* negative size, K % 32 != 0, or K % 128 != 0 for a tiled operand */
+	NH_ERR_NO_DEVICE   = -4, /* no gfx950 device visible */
+	NH_ERR_TOO_LARGE   = -5, /* a dimension exceeds what the launch grid or 32-bit tile indices hold */
+	NH_ERR_ARGUMENT	   = -6 /* any other invalid argument */
+} nh_status;
+
+/* Library / device ------------------------------------------------------------------------------ */
+
+/* Human-readable text for a status returned by any function here (static storage). */
+const char* nh_status_string(int status);
+/* Version of this ABI; bumps when a signature changes. */
+int nh_abi_version(void);
+/* Fills name (NUL-terminated, up to cap bytes) with the device's gcnArchName and *compute_units with its
+ * CU count.  Stands in for the generated nihilus_gpu_properties.hpp (cuda/nihilus_gpu_properties.hpp:28-40). */
+int nh_device_info(char* host_name, int64_t cap, int64_t* host_compute_units, int64_t* host_total_bytes);
+
+/* Arena plumbing for hosts that must not see HIP headers: cudaMalloc / cudaMemcpy wrappers of
+ * cuda/memory_buffer.hpp:78-152.  host_* pointers are host memory. */
+int nh_malloc(void** host_out_dev_ptr, int64_t bytes);
+int nh_free(void* dev_ptr);
+int nh_memcpy_h2d(void* dst_dev, const void* host_src, int64_t bytes, void* stream);
+int nh_memcpy_d2h(void* host_dst, const void* src_dev, int64_t bytes, void* stream);
+int nh_memset(void* dst_dev, int value, int64_t bytes, void* stream);
+/* Blocks until the stream has drained: the cudaDeviceSynchronize after each launch in cuda/cuda_12.hpp:679. */
+int nh_stream_sync(void* stream);
+
+/* Activation quantize -------------------------------------------------------------------------- */
+
+/* quantize_row_q8_0 for M rows (cpu/avx_2.hpp:4439-4489): x fp32 [M][K] row-major -> blocks [M][K/32].
+ * Per block: d = fp16_rne(amax/127), q = int8(round_half_even(x * (127/amax))), amax == 0 -> all zero.
+ * Bit-exact with the reference arithmetic.  K % 32 == 0 (the reference ignores a ragged tail, :4440;
+ * here a ragged K is rejected so no byte is silently dropped). */
+int nh_q8_0_quantize(const float* x, void* xq_blocks, int64_t M, int64_t K, void* stream);
+/* Same values written in the tiled layout (rows padded with zero blocks to a multiple of 32). K % 128 == 0. */
+int nh_q8_0_quantize_tiled(const float* x, void* xq_tiled, int64_t M, int64_t K, void* stream);
+
+/* Layout conversion ---------------------------------------------------------------------------- */
+
+/* Bytes of a [rows x K] matrix: blocks = rows*(K/32)*34 (type_traits<block_q8_0>::total_byte_size,
+ * common/type_traits.hpp:38-61, :185-193); tiled = ceil(rows/32)*(K/128)*4352.  Negative on bad shape. */
+int64_t nh_q8_0_blocks_bytes(int64_t rows, int64_t K);
+int64_t nh_q8_0_tiled_bytes(int64_t rows, int64_t K);
+/* blocks -> tiled (done once per weight at load time, where the reference copies weights into its
+ * device arena: infra/model_parser.hpp:151-154) and back.  Lossless byte permutation. */
+int nh_q8_0_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, void* stream);
+int nh_q8_0_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, void* stream);
+
+/* Mat-vec (decode, eval_time) ------------------------------------------------------------------- */
+
+/* y[n] = sum_b f32(dW[n][b]) * f32(dx[b]) * sum_{j<32} W.qs[n][b][j] * x.qs[b][j]
+ * = vec_dot_q8_0_q8_0<K/32> per output row (cpu/avx_2.hpp:4534-4747), the body the eval_time mul_mat
+ * dispatcher was meant to have (cpu/avx_2.hpp:1371-1444).  Integer block sums are exact; the fp32
+ * accumulation order differs from the CPU's (<= 1e-4 relative L2 over y is the contract, ~1e-7 in practice).
+ * W: N rows, xq: one row of K/32 blocks (always the blocks layout: it is 34*K/32 bytes), y: fp32 [N]. */
+int nh_q8_0_gemv(const void* W_blocks, const void* xq_blocks, float* y, int64_t N, int64_t K, void* stream);
+int nh_q8_0_gemv_tiled(const void* W_tiled, const void* xq_blocks, float* y, int64_t N, int64_t K, void* stream);
+
+/* Mat-mat (prefill, prompt_eval_time) ----------------------------------------------------------- */
+
+/* C[m*N + n] (n fastest, ggml's dst[ir1*nr0 + ir0], cpu/avx_2.hpp:4934) = the same dot for activation
+ * row m: output dims [ne0 = N, ne1 = M] of kernel_traits_old<..., mul_mat, ...> (common/kernel_traits.hpp:393-417),
+ * the body the prompt_eval_time dispatcher was meant to have (cpu/avx_2.hpp:1296-1369).
+ * int8 MFMA (v_mfma_i32_32x32x32_i8) per 32-quant block, fp32 scale application per block. */
+int nh_q8_0_gemm(const void* W_blocks, const void* Aq_blocks, float* C, int64_t M, int64_t N, int64_t K, void* stream);
+int nh_q8_0_gemm_tiled(const void* W_tiled, const void* Aq_tiled, float* C, int64_t M, int64_t N, int64_t K, void* stream);
+
+/* Fused mul_mat: fp32 activations in, fp32 out -------------------------------------------------- */
+
+/* Scratch the fused call needs for the quantized activations (device bytes, 256-byte aligned by the caller). */
+int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K);
+/* quantize(x) then GEMV (M == 1) or GEMM (M > 1) against a tiled weight: the whole
+ * rms_norm-output -> projection step of core_traits.hpp:575-594 / :976-989 as one call. */
+int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Parity instrumentation ------------------------------------------------------------------------ */
+
+/* Per-(m, n, block) int32 sums as the production kernels compute them (same device code path, results
+ * diverted before scaling): sums[(m*N + n)*(K/32) + b].  path 0 = the GEMV kernel's v_dot4 path
+ * (M must be 1), path 1 = the GEMM kernel's MFMA path.  Operands in the blocks layout. */
+int nh_q8_0_debug_block_sums(const void* W_blocks, const void* Aq_blocks, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream);
+
+/* Synthetic inputs (benchmark / test utility) --------------------------------------------------- */
+
+/* Counter-based generator, identical by specification to the CPU checker's: weight blocks with quants uniform in
+ * [-127,127] and d = fp16(|g|*0.01), activations g, g ~ Irwin-Hall(12) standardised.  first_block offsets the
+ * counter so several matrices can be drawn from one seed. */
+int nh_q8_0_fill_weight_blocks(void* blocks, uint64_t seed, int64_t first_block, int64_t n_blocks, void* stream);
+int nh_q8_0_fill_activations(float* x, uint64_t seed, int64_t count, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,354 @@
+// extern "C" surface of the gfx950 Q8_0 library: argument checks, then the launch functions.
+// Nothing here computes; every rejected argument returns a negative nh_status before any launch, so a
+// malformed call can never reach a kernel with shapes the kernel does not expect.
+#include "../../include/nihilus_amd/q8_0_abi.h"
+#include "q8_0_device.h"
+
+#include <cstring>
+
+namespace {
+
+constexpr int64_t MAX_ROWS = int64_t{ 1 } << 30; // row and strip indices are 32-bit inside the kernels
+constexpr int64_t MAX_BLOCKS = int64_t{ 1 } << 35; // blocks per matrix the element-wise kernels can index
+constexpr int64_t MAX_K	   = 49152; // the mat-vec keeps the whole activation row (K + K/8 bytes) in 64 KiB of LDS
+
+inline bool aligned16(const void* p) {
+	return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+inline hipStream_t as_stream(void* s) {
+	return static_cast<hipStream_t>(s);
+}
+inline int from_hip(hipError_t e) {
+	return e == hipSuccess ? NH_OK : static_cast<int>(e);
+}
+
+// Common shape checks: sizes non-negative, K a whole number of blocks (of groups for a tiled operand).
+inline int check_shape(int64_t rows_a, int64_t rows_b, int64_t K, bool tiled) {
+	if (rows_a < 0 || rows_b < 0 || K < 0) {
+		return NH_ERR_SHAPE;
+	}
+	if (K % NH_Q8_0_QK != 0 || (tiled && K % nh::GROUP_K != 0)) {
+		return NH_ERR_SHAPE;
+	}
+	if (rows_a > MAX_ROWS || rows_b > MAX_ROWS || K > MAX_K) {
+		return NH_ERR_TOO_LARGE;
+	}
+	if (rows_a * (K / NH_Q8_0_QK) > MAX_BLOCKS || rows_b * (K / NH_Q8_0_QK) > MAX_BLOCKS) {
+		return NH_ERR_TOO_LARGE; // one thread per four quants, 256 per workgroup, 2^31 workgroups at most
+	}
+	return NH_OK;
+}
+
+// First call on a thread: make sure a gfx950 device is current.  Returns NH_OK or NH_ERR_NO_DEVICE.
+int require_device() {
+	static thread_local int cached = 1; // 1 = not checked yet
+	if (cached != 1) {
+		return cached;
+	}
+	int count = 0;
+	if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+		(void)hipGetLastError();
+		return cached = NH_ERR_NO_DEVICE;
+	}
+	int dev = 0;
+	hipDeviceProp_t prop;
+	if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+		(void)hipGetLastError();
+		return cached = NH_ERR_NO_DEVICE;
+	}
+	if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+		return cached = NH_ERR_NO_DEVICE; // the code object holds gfx950 ISA only
+	}
+	return cached = NH_OK;
+}
+
+} // namespace
+
+#define NH_REQUIRE(cond, code) \
+	do {                       \
+		if (!(cond)) {         \
+			return (code);     \
+		}                      \
+	} while (0)
+#define NH_TRY(expr)        \
+	do {                    \
+		const int rc_ = (expr); \
+		if (rc_ != NH_OK) { \
+			return rc_;     \
+		}                   \
+	} while (0)
+
+extern "C" {
+
+const char* nh_status_string(int status) {
+	switch (status) {
+		case NH_OK:
+			return "ok";
+		case NH_ERR_NULL_POINTER:
+			return "null pointer";
+		case NH_ERR_ALIGNMENT:
+			return "pointer not 16-byte aligned";
+		case NH_ERR_SHAPE:
+			return "bad shape (negative size, K not a multiple of 32, or of 128 for a tiled operand)";
+		case NH_ERR_NO_DEVICE:
+			return "no gfx950 device";
+		case NH_ERR_TOO_LARGE:
+			return "dimension too large";
+		case NH_ERR_ARGUMENT:
+			return "invalid argument";
+		default:
+			return status > 0 ? hipGetErrorString(static_cast<hipError_t>(status)) : "unknown status";
+	}
+}
+
+int nh_abi_version(void) {
+	return 1;
+}
+
+int nh_device_info(char* host_name, int64_t cap, int64_t* host_compute_units, int64_t* host_total_bytes) {
+	NH_TRY(require_device());
+	int dev = 0;
+	hipDeviceProp_t prop;
+	NH_TRY(from_hip(hipGetDevice(&dev)));
+	NH_TRY(from_hip(hipGetDeviceProperties(&prop, dev)));
+	if (host_name && cap > 0) {
+		std::strncpy(host_name, prop.gcnArchName, static_cast<size_t>(cap - 1));
+		host_name[cap - 1] = '\0';
+	}
+	if (host_compute_units) {
+		*host_compute_units = prop.multiProcessorCount;
+	}
+	if (host_total_bytes) {
+		*host_total_bytes = static_cast<int64_t>(prop.totalGlobalMem);
+	}
+	return NH_OK;
+}
+
+int nh_malloc(void** host_out_dev_ptr, int64_t bytes) {
+	NH_REQUIRE(host_out_dev_ptr, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(bytes >= 0, NH_ERR_SHAPE);
+	NH_TRY(require_device());
+	*host_out_dev_ptr = nullptr;
+	if (bytes == 0) {
+		return NH_OK;
+	}
+	return from_hip(hipMalloc(host_out_dev_ptr, static_cast<size_t>(bytes)));
+}
+
+int nh_free(void* dev_ptr) {
+	if (!dev_ptr) {
+		return NH_OK;
+	}
+	return from_hip(hipFree(dev_ptr));
+}
+
+int nh_memcpy_h2d(void* dst_dev, const void* host_src, int64_t bytes, void* stream) {
+	NH_REQUIRE(bytes >= 0, NH_ERR_SHAPE);
+	if (bytes == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(dst_dev && host_src, NH_ERR_NULL_POINTER);
+	NH_TRY(require_device());
+	return from_hip(hipMemcpyAsync(dst_dev, host_src, static_cast<size_t>(bytes), hipMemcpyHostToDevice, as_stream(stream)));
+}
+
+int nh_memcpy_d2h(void* host_dst, const void* src_dev, int64_t bytes, void* stream) {
+	NH_REQUIRE(bytes >= 0, NH_ERR_SHAPE);
+	if (bytes == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(host_dst && src_dev, NH_ERR_NULL_POINTER);
+	NH_TRY(require_device());
+	return from_hip(hipMemcpyAsync(host_dst, src_dev, static_cast<size_t>(bytes), hipMemcpyDeviceToHost, as_stream(stream)));
+}
+
+int nh_memset(void* dst_dev, int value, int64_t bytes, void* stream) {
+	NH_REQUIRE(bytes >= 0, NH_ERR_SHAPE);
+	if (bytes == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(dst_dev, NH_ERR_NULL_POINTER);
+	NH_TRY(require_device());
+	return from_hip(hipMemsetAsync(dst_dev, value, static_cast<size_t>(bytes), as_stream(stream)));
+}
+
+int nh_stream_sync(void* stream) {
+	NH_TRY(require_device());
+	return from_hip(hipStreamSynchronize(as_stream(stream)));
+}
+
+int64_t nh_q8_0_blocks_bytes(int64_t rows, int64_t K) {
+	if (rows < 0 || K < 0 || K % NH_Q8_0_QK != 0) {
+		return NH_ERR_SHAPE;
+	}
+	return rows * (K / NH_Q8_0_QK) * NH_Q8_0_BLOCK_BYTES;
+}
+
+int64_t nh_q8_0_tiled_bytes(int64_t rows, int64_t K) {
+	if (rows < 0 || K < 0 || K % nh::GROUP_K != 0) {
+		return NH_ERR_SHAPE;
+	}
+	return (rows + nh::STRIP_ROWS - 1) / nh::STRIP_ROWS * (K / nh::GROUP_K) * nh::MACRO_BYTES;
+}
+
+int nh_q8_0_quantize(const float* x, void* xq_blocks, int64_t M, int64_t K, void* stream) {
+	NH_TRY(check_shape(M, 0, K, false));
+	if (M == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(x && xq_blocks, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(x) && aligned16(xq_blocks), NH_ERR_ALIGNMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_quantize(x, xq_blocks, M, K, false, as_stream(stream)));
+}
+
+int nh_q8_0_quantize_tiled(const float* x, void* xq_tiled, int64_t M, int64_t K, void* stream) {
+	NH_TRY(check_shape(M, 0, K, true));
+	if (M == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(x && xq_tiled, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(x) && aligned16(xq_tiled), NH_ERR_ALIGNMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_quantize(x, xq_tiled, M, K, true, as_stream(stream)));
+}
+
+int nh_q8_0_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, void* stream) {
+	NH_TRY(check_shape(rows, 0, K, true));
+	if (rows == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(blocks && tiled, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(blocks) && aligned16(tiled), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(blocks != tiled, NH_ERR_ARGUMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_tile(blocks, tiled, rows, K, as_stream(stream)));
+}
+
+int nh_q8_0_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, void* stream) {
+	NH_TRY(check_shape(rows, 0, K, true));
+	if (rows == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(blocks && tiled, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(blocks) && aligned16(tiled), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(blocks != tiled, NH_ERR_ARGUMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_untile(tiled, blocks, rows, K, as_stream(stream)));
+}
+
+static int gemv_common(const void* W, const void* xq, float* y, int64_t N, int64_t K, bool tiled, void* stream) {
+	NH_TRY(check_shape(N, 0, K, tiled));
+	if (N == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(y, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(y), NH_ERR_ALIGNMENT);
+	if (K > 0) {
+		NH_REQUIRE(W && xq, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(W) && aligned16(xq), NH_ERR_ALIGNMENT);
+	}
+	NH_TRY(require_device());
+	return from_hip(nh::launch_gemv(W, xq, y, nullptr, N, K, tiled, as_stream(stream)));
+}
+
+int nh_q8_0_gemv(const void* W_blocks, const void* xq_blocks, float* y, int64_t N, int64_t K, void* stream) {
+	return gemv_common(W_blocks, xq_blocks, y, N, K, false, stream);
+}
+
+int nh_q8_0_gemv_tiled(const void* W_tiled, const void* xq_blocks, float* y, int64_t N, int64_t K, void* stream) {
+	return gemv_common(W_tiled, xq_blocks, y, N, K, true, stream);
+}
+
+static int gemm_common(const void* W, const void* A, float* C, int64_t M, int64_t N, int64_t K, bool tiled, void* stream) {
+	NH_TRY(check_shape(M, N, K, tiled));
+	if (M == 0 || N == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(M <= 65535 * 128, NH_ERR_TOO_LARGE); // grid.y
+	NH_REQUIRE(C, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(C), NH_ERR_ALIGNMENT);
+	if (K > 0) {
+		NH_REQUIRE(W && A, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(W) && aligned16(A), NH_ERR_ALIGNMENT);
+	}
+	NH_TRY(require_device());
+	return from_hip(nh::launch_gemm(W, A, C, nullptr, M, N, K, tiled, as_stream(stream)));
+}
+
+int nh_q8_0_gemm(const void* W_blocks, const void* Aq_blocks, float* C, int64_t M, int64_t N, int64_t K, void* stream) {
+	return gemm_common(W_blocks, Aq_blocks, C, M, N, K, false, stream);
+}
+
+int nh_q8_0_gemm_tiled(const void* W_tiled, const void* Aq_tiled, float* C, int64_t M, int64_t N, int64_t K, void* stream) {
+	return gemm_common(W_tiled, Aq_tiled, C, M, N, K, true, stream);
+}
+
+int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K) {
+	if (M < 0 || K < 0 || K % nh::GROUP_K != 0) {
+		return NH_ERR_SHAPE;
+	}
+	if (M == 1) {
+		return (nh_q8_0_blocks_bytes(1, K) + 255) / 256 * 256;
+	}
+	return (nh_q8_0_tiled_bytes(M, K) + 255) / 256 * 256;
+}
+
+int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
+	NH_TRY(check_shape(M, N, K, true));
+	if (M == 0 || N == 0) {
+		return NH_OK;
+	}
+	const int64_t need = nh_q8_0_mul_mat_workspace_bytes(M, K);
+	NH_REQUIRE(workspace_bytes >= need, NH_ERR_ARGUMENT);
+	if (K > 0) {
+		NH_REQUIRE(workspace && x, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(workspace) && aligned16(x), NH_ERR_ALIGNMENT);
+	}
+	if (M == 1) {
+		NH_TRY(nh_q8_0_quantize(x, workspace, 1, K, stream));
+		return nh_q8_0_gemv_tiled(W_tiled, workspace, y, N, K, stream);
+	}
+	NH_TRY(nh_q8_0_quantize_tiled(x, workspace, M, K, stream));
+	return nh_q8_0_gemm_tiled(W_tiled, workspace, y, M, N, K, stream);
+}
+
+int nh_q8_0_debug_block_sums(const void* W_blocks, const void* Aq_blocks, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream) {
+	NH_TRY(check_shape(M, N, K, false));
+	NH_REQUIRE(path == 0 || path == 1, NH_ERR_ARGUMENT);
+	NH_REQUIRE(path == 1 || M == 1, NH_ERR_ARGUMENT);
+	if (M == 0 || N == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(W_blocks && Aq_blocks && sums, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(W_blocks) && aligned16(Aq_blocks) && aligned16(sums), NH_ERR_ALIGNMENT);
+	NH_TRY(require_device());
+	if (path == 0) {
+		return from_hip(nh::launch_gemv(W_blocks, Aq_blocks, nullptr, sums, N, K, false, as_stream(stream)));
+	}
+	return from_hip(nh::launch_gemm(W_blocks, Aq_blocks, nullptr, sums, M, N, K, false, as_stream(stream)));
+}
+
+int nh_q8_0_fill_weight_blocks(void* blocks, uint64_t seed, int64_t first_block, int64_t n_blocks, void* stream) {
+	NH_REQUIRE(n_blocks >= 0 && first_block >= 0, NH_ERR_SHAPE);
+	if (n_blocks == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(n_blocks <= MAX_BLOCKS, NH_ERR_TOO_LARGE);
+	NH_REQUIRE(blocks, NH_ERR_NULL_POINTER);
+	NH_REQUIRE((reinterpret_cast<uintptr_t>(blocks) & 1u) == 0, NH_ERR_ALIGNMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_fill_weights(blocks, seed, first_block, n_blocks, as_stream(stream)));
+}
+
+int nh_q8_0_fill_activations(float* x, uint64_t seed, int64_t count, void* stream) {
+	NH_REQUIRE(count >= 0, NH_ERR_SHAPE);
+	if (count == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(x, NH_ERR_NULL_POINTER);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_fill_activations(x, seed, count, as_stream(stream)));
+}
+
+} // extern "C"

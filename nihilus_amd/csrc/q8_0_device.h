@@ -1,0 +1,67 @@
+// Device-side helpers shared by the gfx950 Q8_0 kernels: layout constants, fp16 scale conversion,
+// the packed int8 dot, and the launch functions each translation unit exports to the C ABI file.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nh {
+
+constexpr int QK			= 32; // quants per block (Q_SIZE, common/data_types.hpp:28)
+constexpr int BLOCK_BYTES	= 34; // fp16 d + 32 int8 (common/data_types.hpp:38-44)
+constexpr int STRIP_ROWS	= 32; // rows per tiled strip = MFMA 32x32x32 operand rows
+constexpr int GROUP_BLOCKS	= 4; // blocks per macro-tile along K
+constexpr int GROUP_K		= GROUP_BLOCKS * QK; // 128
+constexpr int TILE_BYTES	= 1024; // 32 rows x 32 quants, in MFMA operand order
+constexpr int MACRO_BYTES	= GROUP_BLOCKS * TILE_BYTES + STRIP_ROWS * GROUP_BLOCKS * 2; // 4352 = 32 rows x 4 blocks x 34
+constexpr int MACRO_D_OFFSET = GROUP_BLOCKS * TILE_BYTES; // 4096
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// fp16 bits -> fp32, exact (v_cvt_f32_f16; fp16 subnormals are honoured: the kernel's float mode keeps them).
+__device__ __forceinline__ float half_bits_to_float(uint16_t h) {
+	return __half2float(__ushort_as_half(h));
+}
+// fp32 -> fp16 bits, round to nearest even, subnormals kept, overflow to inf (v_cvt_f16_f32).
+__device__ __forceinline__ uint16_t float_to_half_bits(float f) {
+	return __half_as_ushort(__float2half_rn(f));
+}
+// c + sum of four int8 x int8 products, exact (v_dot4_i32_i8).
+__device__ __forceinline__ int dot4(int a, int b, int c) {
+	return __builtin_amdgcn_sdot4(a, b, c, false);
+}
+__device__ __forceinline__ int dot16(v4i a, v4i b) {
+	int s = dot4(a.x, b.x, 0);
+	s	  = dot4(a.y, b.y, s);
+	s	  = dot4(a.z, b.z, s);
+	return dot4(a.w, b.w, s);
+}
+// 16 bytes from an address that is only 2-byte aligned (the qs field of a packed 34-byte block).
+__device__ __forceinline__ v4i load16_unaligned(const uint8_t* p) {
+	v4i v;
+	__builtin_memcpy(&v, p, 16);
+	return v;
+}
+__device__ __forceinline__ uint16_t load_u16(const uint8_t* p) {
+	return *reinterpret_cast<const uint16_t*>(p);
+}
+
+// Byte offset of macro-tile (strip, group) in a tiled matrix with `groups` = K/128 groups per strip.
+__device__ __host__ __forceinline__ int64_t macro_offset(int64_t strip, int64_t group, int64_t groups) {
+	return (strip * groups + group) * MACRO_BYTES;
+}
+
+// ---- launch functions (defined one per .hip file, called from q8_0_abi.hip after argument checks) ----
+
+hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s);
+hipError_t launch_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, hipStream_t s);
+hipError_t launch_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, hipStream_t s);
+hipError_t launch_fill_weights(void* blocks, uint64_t seed, int64_t first_block, int64_t n_blocks, hipStream_t s);
+hipError_t launch_fill_activations(float* x, uint64_t seed, int64_t count, hipStream_t s);
+// sums == nullptr: production; otherwise the same kernel diverts the per-block int32 sums to `sums` and leaves y alone.
+hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* sums, int64_t N, int64_t K, bool tiled, hipStream_t s);
+hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s);
+
+} // namespace nh

@@ -1,0 +1,85 @@
+// Activation quantize, fp32 -> Q8_0, for gfx950.
+//
+// Restates quantize_row_q8_0 (reference cpu/avx_2.hpp:4439-4489) with bit-exact results:
+//   amax = max|x_i| over 32 values; d = fp16_rne(amax / 127.f) with an IEEE fp32 divide;
+//   id = amax != 0 ? 127.f / amax : 0;  q_i = int8(round_half_even(fl32(x_i * id))).
+// The multiply, the rounding and the divide are kept as separate correctly rounded fp32 operations
+// (__fmul_rn / __fdiv_rn / v_rndne_f32): contracting x*id into anything else would change ties.
+//
+// Memory-bound: 4 bytes read + 1.0625 bytes written per element.  Eight lanes share one block, each
+// loads one float4 (a wavefront reads 1 KiB contiguous), the block maximum is a three-step
+// cross-lane max inside the 8-lane group.
+#include "q8_0_device.h"
+
+namespace nh {
+
+template<bool TILED> __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, uint8_t* __restrict__ out, int64_t M, int64_t rows_out, int64_t K) {
+	const int64_t nb	= K / QK;
+	const int64_t t		= static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+	const int64_t blk	= t >> 3; // block index over rows_out * nb
+	const int j			= static_cast<int>(t & 7); // which float4 of the block
+	const bool in_range = blk < rows_out * nb; // whole 8-lane groups agree, so the shuffles below stay converged per group
+	const int64_t m		= in_range ? blk / nb : 0;
+	const int64_t b		= in_range ? blk - m * nb : 0;
+
+	float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+	if (in_range && m < M) {
+		v = *reinterpret_cast<const float4*>(x + m * K + b * QK + 4 * j);
+	}
+	float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+	amax	   = fmaxf(amax, __shfl_xor(amax, 1));
+	amax	   = fmaxf(amax, __shfl_xor(amax, 2));
+	amax	   = fmaxf(amax, __shfl_xor(amax, 4));
+
+	const float d	  = __fdiv_rn(amax, 127.0f);
+	const float id	  = (amax != 0.0f) ? __fdiv_rn(127.0f, amax) : 0.0f;
+	const uint16_t dh = float_to_half_bits(d);
+
+	auto q8 = [id](float f) -> uint32_t {
+		int q = static_cast<int>(rintf(__fmul_rn(f, id))); // v_rndne_f32: ties to even
+		q	  = max(-128, min(127, q)); // the reference's saturating packs; never active for finite input
+		return static_cast<uint32_t>(q) & 0xFFu;
+	};
+	const uint32_t packed = q8(v.x) | (q8(v.y) << 8) | (q8(v.z) << 16) | (q8(v.w) << 24);
+
+	if (!in_range) {
+		return;
+	}
+	if constexpr (TILED) {
+		const int64_t strip = m / STRIP_ROWS;
+		const int r			= static_cast<int>(m % STRIP_ROWS);
+		const int64_t g		= b / GROUP_BLOCKS;
+		const int tq		= static_cast<int>(b % GROUP_BLOCKS);
+		uint8_t* macro		= out + macro_offset(strip, g, K / GROUP_K);
+		const int lane		= r + 32 * (j >> 2); // quants 0..15 live in lanes 0..31, 16..31 in lanes 32..63
+		*reinterpret_cast<uint32_t*>(macro + tq * TILE_BYTES + 16 * lane + 4 * (j & 3)) = packed;
+		if (j == 0) {
+			*reinterpret_cast<uint16_t*>(macro + MACRO_D_OFFSET + 8 * r + 2 * tq) = dh;
+		}
+	} else {
+		uint8_t* o = out + blk * BLOCK_BYTES;
+		// the qs field sits at a 2-byte-aligned address: two half-word stores per lane
+		*reinterpret_cast<uint16_t*>(o + 2 + 4 * j)		= static_cast<uint16_t>(packed & 0xFFFFu);
+		*reinterpret_cast<uint16_t*>(o + 2 + 4 * j + 2) = static_cast<uint16_t>(packed >> 16);
+		if (j == 0) {
+			*reinterpret_cast<uint16_t*>(o) = dh;
+		}
+	}
+}
+
+hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s) {
+	const int64_t rows_out = tiled ? (M + STRIP_ROWS - 1) / STRIP_ROWS * STRIP_ROWS : M;
+	const int64_t threads  = rows_out * (K / QK) * 8;
+	if (threads == 0) {
+		return hipSuccess;
+	}
+	const int64_t grid = (threads + 255) / 256;
+	if (tiled) {
+		quantize_kernel<true><<<dim3(static_cast<unsigned>(grid)), dim3(256), 0, s>>>(x, static_cast<uint8_t*>(out), M, rows_out, K);
+	} else {
+		quantize_kernel<false><<<dim3(static_cast<unsigned>(grid)), dim3(256), 0, s>>>(x, static_cast<uint8_t*>(out), M, rows_out, K);
+	}
+	return hipGetLastError();
+}
+
+} // namespace nh

@@ -1,0 +1,127 @@
+"""Host-side wrappers of the Q8_0 path for callers that hold torch tensors.
+
+torch is used for device memory and streams only; every operation below is one call through the C ABI
+(``include/nihilus_amd/q8_0_abi.h``).  Names follow the reference: ``quantize_row_q8_0``
+(cpu/avx_2.hpp:4439-4489), ``mul_mat`` (kernel_types::mul_mat, cpu/avx_2.hpp:1296-1444).  Q8_0 data is a
+``torch.uint8`` tensor: "blocks" = rows of packed 34-byte block_q8_0, "tiled" = the device layout
+described in the ABI header.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+QK = 32
+BLOCK_BYTES = 34
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, dtype: torch.dtype, name: str) -> torch.Tensor:
+    if not (t.is_cuda and t.dtype == dtype and t.is_contiguous()):
+        raise TypeError(f"{name} must be a contiguous {dtype} tensor on the GPU")
+    return t
+
+
+def blocks_bytes(rows: int, k: int) -> int:
+    n = _lib.lib().nh_q8_0_blocks_bytes(rows, k)
+    _lib.check("nh_q8_0_blocks_bytes", n if n < 0 else 0)
+    return n
+
+
+def tiled_bytes(rows: int, k: int) -> int:
+    n = _lib.lib().nh_q8_0_tiled_bytes(rows, k)
+    _lib.check("nh_q8_0_tiled_bytes", n if n < 0 else 0)
+    return n
+
+
+def quantize_row_q8_0(x: torch.Tensor, tiled: bool = False) -> torch.Tensor:
+    """x fp32 [M, K] (or [K]) -> uint8 blocks [M, K/32*34] (or the tiled byte stream)."""
+    x = _dev(x, torch.float32, "x")
+    x2 = x.reshape(1, -1) if x.dim() == 1 else x
+    m, k = x2.shape
+    if tiled:
+        out = torch.empty(tiled_bytes(m, k), dtype=torch.uint8, device=x.device)
+        _lib.check("nh_q8_0_quantize_tiled", _lib.lib().nh_q8_0_quantize_tiled(x2.data_ptr(), out.data_ptr(), m, k, _stream()))
+        return out
+    out = torch.empty((m, blocks_bytes(1, k)), dtype=torch.uint8, device=x.device)
+    _lib.check("nh_q8_0_quantize", _lib.lib().nh_q8_0_quantize(x2.data_ptr(), out.data_ptr(), m, k, _stream()))
+    return out
+
+
+def tile(blocks: torch.Tensor, rows: int, k: int) -> torch.Tensor:
+    blocks = _dev(blocks, torch.uint8, "blocks")
+    if blocks.numel() != blocks_bytes(rows, k):
+        raise ValueError("blocks tensor does not hold rows*(k/32) blocks")
+    out = torch.empty(tiled_bytes(rows, k), dtype=torch.uint8, device=blocks.device)
+    _lib.check("nh_q8_0_tile", _lib.lib().nh_q8_0_tile(blocks.data_ptr(), out.data_ptr(), rows, k, _stream()))
+    return out
+
+
+def untile(tiled: torch.Tensor, rows: int, k: int) -> torch.Tensor:
+    tiled = _dev(tiled, torch.uint8, "tiled")
+    if tiled.numel() != tiled_bytes(rows, k):
+        raise ValueError("tiled tensor has the wrong size for rows x k")
+    out = torch.empty(blocks_bytes(rows, k), dtype=torch.uint8, device=tiled.device)
+    _lib.check("nh_q8_0_untile", _lib.lib().nh_q8_0_untile(tiled.data_ptr(), out.data_ptr(), rows, k, _stream()))
+    return out
+
+
+def gemv(w: torch.Tensor, xq_blocks: torch.Tensor, n: int, k: int, tiled: bool) -> torch.Tensor:
+    w, xq_blocks = _dev(w, torch.uint8, "w"), _dev(xq_blocks, torch.uint8, "xq_blocks")
+    if w.numel() != (tiled_bytes(n, k) if tiled else blocks_bytes(n, k)) or xq_blocks.numel() != blocks_bytes(1, k):
+        raise ValueError("operand sizes do not match n x k")
+    y = torch.empty(n, dtype=torch.float32, device=w.device)
+    fn = "nh_q8_0_gemv_tiled" if tiled else "nh_q8_0_gemv"
+    _lib.check(fn, getattr(_lib.lib(), fn)(w.data_ptr(), xq_blocks.data_ptr(), y.data_ptr(), n, k, _stream()))
+    return y
+
+
+def gemm(w: torch.Tensor, aq: torch.Tensor, m: int, n: int, k: int, tiled: bool) -> torch.Tensor:
+    w, aq = _dev(w, torch.uint8, "w"), _dev(aq, torch.uint8, "aq")
+    size = tiled_bytes if tiled else blocks_bytes
+    if w.numel() != size(n, k) or aq.numel() != size(m, k):
+        raise ValueError("operand sizes do not match m x n x k")
+    c = torch.empty((m, n), dtype=torch.float32, device=w.device)
+    fn = "nh_q8_0_gemm_tiled" if tiled else "nh_q8_0_gemm"
+    _lib.check(fn, getattr(_lib.lib(), fn)(w.data_ptr(), aq.data_ptr(), c.data_ptr(), m, n, k, _stream()))
+    return c
+
+
+def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 activations [M, K] x tiled Q8_0 weight [N, K] -> fp32 [M, N]: quantize + GEMV/GEMM."""
+    w_tiled, x = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(x, torch.float32, "x")
+    x2 = x.reshape(1, -1) if x.dim() == 1 else x
+    m = x2.shape[0]
+    if x2.shape[1] != k or w_tiled.numel() != tiled_bytes(n, k):
+        raise ValueError("operand sizes do not match m x n x k")
+    need = _lib.lib().nh_q8_0_mul_mat_workspace_bytes(m, k)
+    _lib.check("nh_q8_0_mul_mat_workspace_bytes", need if need < 0 else 0)
+    if workspace is None:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
+    y = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    _lib.check("nh_q8_0_mul_mat", _lib.lib().nh_q8_0_mul_mat(w_tiled.data_ptr(), x2.data_ptr(), y.data_ptr(), m, n, k, workspace.data_ptr(), workspace.numel(), _stream()))
+    return y
+
+
+def debug_block_sums(w_blocks: torch.Tensor, aq_blocks: torch.Tensor, m: int, n: int, k: int, path: int) -> torch.Tensor:
+    """int32 [m, n, k/32] block sums from the GEMV (path 0) or MFMA (path 1) kernel."""
+    sums = torch.empty((m, n, k // QK), dtype=torch.int32, device=w_blocks.device)
+    _lib.check("nh_q8_0_debug_block_sums", _lib.lib().nh_q8_0_debug_block_sums(w_blocks.data_ptr(), aq_blocks.data_ptr(), sums.data_ptr(), m, n, k, path, _stream()))
+    return sums
+
+
+def fill_weight_blocks(seed: int, n: int, k: int, first_block: int = 0, device="cuda") -> torch.Tensor:
+    nblk = n * (k // QK)
+    w = torch.empty(nblk * BLOCK_BYTES, dtype=torch.uint8, device=device)
+    _lib.check("nh_q8_0_fill_weight_blocks", _lib.lib().nh_q8_0_fill_weight_blocks(w.data_ptr(), seed, first_block, nblk, _stream()))
+    return w
+
+
+def fill_activations(seed: int, count: int, device="cuda") -> torch.Tensor:
+    x = torch.empty(count, dtype=torch.float32, device=device)
+    _lib.check("nh_q8_0_fill_activations", _lib.lib().nh_q8_0_fill_activations(x.data_ptr(), seed, count, _stream()))
+    return x

@@ -1,0 +1,88 @@
+"""GPU parity: decode mat-vec vs the CPU restatement.
+
+int32 block sums bit-exact; fp32 y within 1e-4 relative L2 of vec_dot_q8_0_q8_0<K/32> in the reference's
+summation order (the GPU sums in a different order).
+"""
+import numpy as np
+import pytest
+
+from helpers import REL_L2_TOL, random_blocks, rel_l2, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336), (1024, 4096), (96, 512), (33, 128), (1, 128), (31, 256), (257, 8192)]
+
+
+def _inputs(oracle, n, k, seed):
+    w = oracle.fill_weights(seed, n, k)
+    x = oracle.fill_activations(seed, k)
+    return w, x, oracle.quantize_rows(x)[0]
+
+
+@pytest.mark.parametrize("n,k", SHAPES)
+def test_gemv_tiled_and_blocks(q8, oracle, n, k):
+    w, x, xq = _inputs(oracle, n, k, seed=n * 131 + k)
+    want = oracle.gemv(w, xq, n, k)
+    wd, xqd = to_dev(w), to_dev(xq)
+    y_blocks = to_host(q8.gemv(wd, xqd, n, k, tiled=False))
+    y_tiled = to_host(q8.gemv(q8.tile(wd, n, k), xqd, n, k, tiled=True))
+    assert rel_l2(y_blocks, want) <= REL_L2_TOL
+    assert rel_l2(y_tiled, want) <= REL_L2_TOL
+    # both layouts hold the same values and the kernel sums them in the same order
+    assert np.array_equal(y_blocks, y_tiled)
+    # far tighter than the contract in practice
+    assert rel_l2(y_tiled, oracle.gemv_f64(w, xq, n, k)) < 5e-6
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (96, 512), (33, 160), (5, 32)])
+def test_gemv_block_sums_exact(q8, oracle, n, k):
+    w, x, xq = _inputs(oracle, n, k, seed=5)
+    want = oracle.block_sums_gemv(w, xq, n, k)
+    got = to_host(q8.debug_block_sums(to_dev(w), to_dev(xq), 1, n, k, path=0))[0]
+    assert np.array_equal(got, want)
+
+
+def test_gemv_ragged_k_blocks_layout(q8, oracle):
+    # K a multiple of 32 but not of 128: only the blocks layout takes it
+    rng = np.random.default_rng(3)
+    for n, k in [(40, 32), (40, 96), (7, 608)]:
+        w = random_blocks(rng, n, k)
+        xq = oracle.quantize_rows(rng.standard_normal(k).astype(np.float32))[0]
+        got = to_host(q8.gemv(to_dev(w), to_dev(xq), n, k, tiled=False))
+        assert rel_l2(got, oracle.gemv(w, xq, n, k)) <= REL_L2_TOL
+
+
+def test_gemv_extreme_quants_and_unit_scales(q8, oracle):
+    n, k = 64, 256
+    nb = k // 32
+    one = np.float16(1.0).view(np.uint16)
+    # all +-127 against all 127, d = 1: y is an exact integer, 127*127*k (with sign)
+    sign = np.where(np.arange(n) % 2 == 0, 127, -127).astype(np.int8)
+    w = oracle.pack_blocks(np.full(n * nb, one), np.repeat(sign[:, None], k, axis=1))
+    xq = oracle.pack_blocks(np.full(nb, one), np.full(k, 127, dtype=np.int8))
+    y = to_host(q8.gemv(to_dev(w), to_dev(xq), n, k, tiled=False))
+    assert np.array_equal(y, sign.astype(np.float32) * 127.0 * k)
+    sums = to_host(q8.debug_block_sums(to_dev(w), to_dev(xq), 1, n, k, path=0))[0]
+    assert np.array_equal(sums, np.repeat((sign.astype(np.int32) * 127 * 32)[:, None], nb, axis=1))
+
+
+def test_gemv_errors(q8):
+    import torch
+
+    from nihilus_amd import _lib
+
+    lib = _lib.lib()
+    w = torch.zeros(34 * 4 * 32, dtype=torch.uint8, device="cuda")
+    xq = torch.zeros(34 * 4, dtype=torch.uint8, device="cuda")
+    y = torch.full((32,), 7.0, dtype=torch.float32, device="cuda")
+    assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 0, 128, None) == 0
+    assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 100, None) == -3
+    assert lib.nh_q8_0_gemv_tiled(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 96, None) == -3
+    assert lib.nh_q8_0_gemv(None, xq.data_ptr(), y.data_ptr(), 32, 128, None) == -1
+    assert lib.nh_q8_0_gemv(w.data_ptr() + 2, xq.data_ptr(), y.data_ptr(), 32, 128, None) == -2
+    assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 1 << 20, None) == -5
+    torch.cuda.synchronize()
+    assert bool((y == 7.0).all())  # rejected calls wrote nothing
+    assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 0, None) == 0  # empty dot product
+    torch.cuda.synchronize()
+    assert bool((y == 0.0).all())
