@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the Q8_0 mat-mul hot path on one MI355X.
+
+Workload (the configuration the metric is quoted on): the LLaMA-3-8B FFN decode mat-vecs at batch 1 --
+gate and up, Q8_0 W [14336 x 4096], and down, Q8_0 W [4096 x 14336] -- with the activation quantize inside
+the step.  One step = quantize(x[4096]) -> gate, up ; quantize(h[14336]) -> down, enqueued by one native
+batch call.  Steps rotate over `--layers` distinct weight sets (default 16 x 187 MB = 3 GB) so that every
+byte comes from HBM and not from the 256 MB last-level cache.  Inputs are resident in HBM before the timed
+region; synthetic data from the library's counter-based generator (seed 0).
+
+Prints ONE JSON line.  `value` = algorithmic bytes per step / wall time per step.  `roofline` is for the
+dominant kernel (the tiled mat-vec): algorithmic bytes per launch / its average duration, measured live with
+start/stop timestamps carried in each launch's own dispatch packet.  `cpu_baseline` is the AVX2 restatement
+of the reference arithmetic on the host's cores (a reported number, not the target).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+GATE_N, HIDDEN, FFN = 14336, 4096, 14336
+
+
+def gemv_bytes(n: int, k: int, with_quantize: bool) -> int:
+    """Algorithmic bytes of one mat-vec: weights + quantized x + fp32 y (+ fp32 x when the quantize is counted)."""
+    nb = k // 32
+    return n * nb * 34 + nb * 34 + 4 * n + (4 * k if with_quantize else 0)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--layers", type=int, default=16, help="distinct weight sets rotated through (HBM, not cache)")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
+    ap.add_argument("--roofline-steps", type=int, default=0, help="steps of the per-kernel timing pass (default: min(steps, 1000))")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from nihilus_amd import _lib, q8_0
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        return 3
+    lib = _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    # ---------------------------------------------------------------- inputs, resident in HBM
+    L = max(1, args.layers)
+    nb_h, nb_f = HIDDEN // 32, FFN // 32
+    layers = []
+    first = 0
+    for _ in range(L):
+        mats = []
+        for n, k in ((GATE_N, HIDDEN), (GATE_N, HIDDEN), (HIDDEN, FFN)):
+            blocks = q8_0.fill_weight_blocks(0, n, k, first_block=first)
+            first += n * (k // 32)
+            mats.append(q8_0.tile(blocks, n, k))
+            del blocks
+        layers.append(mats)
+    x = q8_0.fill_activations(0, HIDDEN)  # FFN input (post-norm hidden state), fp32 N(0,1)
+    h = q8_0.fill_activations(1, FFN)  # down-projection input, fp32 N(0,1)
+    y_gate = torch.empty(GATE_N, dtype=torch.float32, device=dev)
+    y_up = torch.empty(GATE_N, dtype=torch.float32, device=dev)
+    y_down = torch.empty(HIDDEN, dtype=torch.float32, device=dev)
+    ws_bytes = max(lib.nh_q8_0_mul_mat_workspace_bytes(1, HIDDEN), lib.nh_q8_0_mul_mat_workspace_bytes(1, FFN))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+    OpArr = _lib.MulMatOp * 3
+    op_lists = []
+    for mats in layers:
+        ops = OpArr()
+        ops[0] = _lib.MulMatOp(mats[0].data_ptr(), x.data_ptr(), y_gate.data_ptr(), 1, GATE_N, HIDDEN, 0, 0)
+        ops[1] = _lib.MulMatOp(mats[1].data_ptr(), x.data_ptr(), y_up.data_ptr(), 1, GATE_N, HIDDEN, 1, 0)
+        ops[2] = _lib.MulMatOp(mats[2].data_ptr(), h.data_ptr(), y_down.data_ptr(), 1, HIDDEN, FFN, 0, 0)
+        op_lists.append(ops)
+
+    batch = lib.nh_q8_0_mul_mat_batch
+    ws_ptr, ws_n = ws.data_ptr(), ws.numel()
+
+    def run_steps(count: int, start: int = 0) -> None:
+        for i in range(start, start + count):
+            rc = batch(op_lists[i % L], 3, ws_ptr, ws_n, stream)
+            if rc != 0:
+                _lib.check("nh_q8_0_mul_mat_batch", rc)
+
+    # quantize reads 4K bytes of fp32 x once per distinct activation: x for gate+up, h for down
+    step_bytes = gemv_bytes(GATE_N, HIDDEN, True) + gemv_bytes(GATE_N, HIDDEN, False) + gemv_bytes(HIDDEN, FFN, True)
+
+    # ---------------------------------------------------------------- warm-up, then EXACTLY --steps timed steps
+    run_steps(args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_steps(args.steps, start=args.warmup)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    sec_per_step = (t1 - t0) / args.steps
+    value = step_bytes / sec_per_step / 1e9
+
+    # ---------------------------------------------------------------- dominant kernel, timed per launch
+    rsteps = args.roofline_steps or min(args.steps, 1000)
+    _lib.check("nh_profile_begin", lib.nh_profile_begin(1, 3 * rsteps))
+    run_steps(rsteps, start=args.warmup + args.steps)
+    tot, cnt, mn, mx = C.c_double(), C.c_int64(), C.c_double(), C.c_double()
+    _lib.check("nh_profile_end", lib.nh_profile_end(C.byref(tot), C.byref(cnt), C.byref(mn), C.byref(mx)))
+    launch_bytes = (2 * gemv_bytes(GATE_N, HIDDEN, False) + gemv_bytes(HIDDEN, FFN, False)) / 3.0
+    avg_ms = tot.value / max(1, cnt.value)
+    achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
+
+    # sanity: the last step's outputs are finite (a wrong kernel would usually show up here first)
+    finite = bool(torch.isfinite(y_gate).all() and torch.isfinite(y_up).all() and torch.isfinite(y_down).all())
+
+    result = {
+        "metric": "Q8_0 GEMV HBM GB/s (% of peak) + LLaMA-3-8B-shape decode tok/s, 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec_per_step * 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": "LLaMA-3-8B FFN decode GEMVs, batch 1: gate+up Q8_0 [14336x4096], down Q8_0 [4096x14336], activation quantize included",
+            "weight_sets_rotated": L,
+            "bytes_per_step": step_bytes,
+            "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+            "outputs_finite": finite,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "nh::gemv_kernel<4, true, false> (tiled mat-vec)",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "bytes_per_launch": launch_bytes,
+            "avg_launch_us": round(avg_ms * 1e3, 3),
+            "min_launch_us": round(mn.value * 1e3, 3),
+            "max_launch_us": round(mx.value * 1e3, 3),
+            "launches_timed": cnt.value,
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+
+    print(json.dumps(result))
+    return 0
+
+
+def cpu_baseline(budget_s: float) -> dict:
+    """The AVX2 restatement (oracle/q8_0_avx2.c) on the host's cores: quantize + mat-vec over rotating weights."""
+    import numpy as np
+
+    import oracle as O  # the checker, used here only as the reported CPU baseline
+
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = max(1, min(16, cores))  # the GPU box gives one job 16 cores' worth of CPU
+    n_sets = 3
+    w_gate = np.concatenate([O.fill_weights(0, GATE_N, HIDDEN, first_block=i * GATE_N * (HIDDEN // 32)) for i in range(n_sets)])
+    w_down = np.concatenate([O.fill_weights(7, HIDDEN, FFN, first_block=i * HIDDEN * (FFN // 32)) for i in range(n_sets)])
+    x = O.fill_activations(0, HIDDEN)
+    h = O.fill_activations(1, FFN)
+    # short calibration, then a bounded sample
+    t_g = O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, threads, 3, pin=False)
+    t_d = O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, threads, 3, pin=False)
+    per_pass = 2 * t_g + t_d
+    passes = int(max(3, min(400, budget_s / max(per_pass, 1e-6))))
+    t_g = O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, threads, 2 * passes, pin=False)
+    t_d = O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, threads, passes, pin=False)
+    sec = 2 * t_g + t_d
+    nbytes = 2 * gemv_bytes(GATE_N, HIDDEN, True) + gemv_bytes(HIDDEN, FFN, True)
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {
+        "value": round(nbytes / sec / 1e9, 2),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{passes} passes of the same FFN step (gate, up, down mat-vecs + quantize) over {n_sets} rotating weight sets, "
+        f"AVX2/FMA/F16C restatement of the reference arithmetic, {threads} threads, rows claimed through an atomic chunk counter",
+        "cpu_model": model,
+        "ms_per_step": round(sec * 1e3, 3),
+    }
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -116,6 +116,31 @@ int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K);
  * rms_norm-output -> projection step of core_traits.hpp:575-594 / :976-989 as one call. */
 int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* One entry of a batch: y[M][N] = mul_mat(W_tiled [N x K], x fp32 [M][K]).  reuse_quantized_x != 0 lets the runner
+ * skip the quantize when the previous entry quantized the same x pointer with the same M and K (q/k/v share the
+ * normed hidden state, gate/up share the FFN input: infra/core_traits.hpp:575-594, :976-986). */
+typedef struct nh_q8_0_mul_mat_op {
+	const void* W_tiled;
+	const float* x;
+	float* y;
+	int64_t M, N, K;
+	int32_t reuse_quantized_x;
+	int32_t reserved;
+} nh_q8_0_mul_mat_op;
+/* Enqueues `count` mul_mat operations in order on one stream from native code: one call per decode step instead
+ * of one per projection (the per-block fold of cuda/thread_pool.hpp:46-67 over the three mega cores).  host_ops is
+ * host memory, read before return.  workspace must hold the largest nh_q8_0_mul_mat_workspace_bytes(M, K) of the
+ * list; entries run in stream order, so sharing it is safe.  All entries are validated before the first launch. */
+int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Per-kernel timing (instrumentation) ----------------------------------------------------------- */
+
+/* kernel_kind: 0 = quantize, 1 = mat-vec, 2 = mat-mat.  Between begin and end every launch of that kind (up to
+ * max_launches) records GPU timestamps at the kernel's own start and end.  nh_profile_end waits for them and
+ * returns the summed, smallest and largest kernel durations in milliseconds.  Process-wide; not for concurrent use. */
+int nh_profile_begin(int kernel_kind, int64_t max_launches);
+int nh_profile_end(double* host_total_ms, int64_t* host_launches, double* host_min_ms, double* host_max_ms);
+
 /* Parity instrumentation ------------------------------------------------------------------------ */
 
 /* Per-(m, n, block) int32 sums as the production kernels compute them (same device code path, results

@@ -35,10 +35,19 @@ SIGNATURES = {
     "nh_q8_0_gemm_tiled": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "nh_q8_0_mul_mat_workspace_bytes": (_i64, [_i64, _i64]),
     "nh_q8_0_mul_mat": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "nh_q8_0_mul_mat_batch": (_int, [_vp, _i64, _vp, _i64, _vp]),
+    "nh_profile_begin": (_int, [_int, _i64]),
+    "nh_profile_end": (_int, [C.POINTER(C.c_double), C.POINTER(_i64), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "nh_q8_0_debug_block_sums": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "nh_q8_0_fill_weight_blocks": (_int, [_vp, _u64, _i64, _i64, _vp]),
     "nh_q8_0_fill_activations": (_int, [_vp, _u64, _i64, _vp]),
 }
+
+
+class MulMatOp(C.Structure):
+    """nh_q8_0_mul_mat_op"""
+
+    _fields_ = [("W_tiled", _vp), ("x", _vp), ("y", _vp), ("M", _i64), ("N", _i64), ("K", _i64), ("reuse_quantized_x", C.c_int32), ("reserved", C.c_int32)]
 
 
 class Q8Error(RuntimeError):

@@ -2,6 +2,7 @@
 // the packed int8 dot, and the launch functions each translation unit exports to the C ABI file.
 #pragma once
 
+#include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -51,6 +52,26 @@ __device__ __forceinline__ uint16_t load_u16(const uint8_t* p) {
 // Byte offset of macro-tile (strip, group) in a tiled matrix with `groups` = K/128 groups per strip.
 __device__ __host__ __forceinline__ int64_t macro_offset(int64_t strip, int64_t group, int64_t groups) {
 	return (strip * groups + group) * MACRO_BYTES;
+}
+
+// ---- per-kernel timing (opt-in instrumentation, see q8_0_profile.hip) ----
+
+enum kernel_kind : int { KIND_QUANTIZE = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_COUNT = 3 };
+
+// When timing is on for `kind` and the event pool has room, hands out an event pair for the next launch.
+bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop);
+
+// Every compute kernel goes through here: a plain launch, or, while timing is on, a launch whose dispatch
+// packet records GPU timestamps at the kernel's own start and end (what a kernel trace reports as its duration).
+template<typename Kernel, typename... Args>
+inline hipError_t launch_kernel(int kind, Kernel kernel, dim3 grid, dim3 block, size_t shmem, hipStream_t s, Args... args) {
+	hipEvent_t e0, e1;
+	if (profile_next(kind, &e0, &e1)) {
+		hipExtLaunchKernelGGL(kernel, grid, block, static_cast<uint32_t>(shmem), s, e0, e1, 0, args...);
+	} else {
+		kernel<<<grid, block, shmem, s>>>(args...);
+	}
+	return hipGetLastError();
 }
 
 // ---- launch functions (defined one per .hip file, called from q8_0_abi.hip after argument checks) ----

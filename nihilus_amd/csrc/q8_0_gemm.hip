@@ -171,13 +171,13 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 		if (sums) {
 			gemm_kernel<true, true><<<grid, dim3(GEMM_THREADS), 0, s>>>(w, a, C, sums, m, n, k);
 		} else {
-			gemm_kernel<true, false><<<grid, dim3(GEMM_THREADS), 0, s>>>(w, a, C, sums, m, n, k);
+			return launch_kernel(KIND_GEMM, gemm_kernel<true, false>, grid, dim3(GEMM_THREADS), 0, s, w, a, C, sums, m, n, k);
 		}
 	} else {
 		if (sums) {
 			gemm_kernel<false, true><<<grid, dim3(GEMM_THREADS), 0, s>>>(w, a, C, sums, m, n, k);
 		} else {
-			gemm_kernel<false, false><<<grid, dim3(GEMM_THREADS), 0, s>>>(w, a, C, sums, m, n, k);
+			return launch_kernel(KIND_GEMM, gemm_kernel<false, false>, grid, dim3(GEMM_THREADS), 0, s, w, a, C, sums, m, n, k);
 		}
 	}
 	return hipGetLastError();

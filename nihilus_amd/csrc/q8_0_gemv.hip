@@ -126,10 +126,9 @@ template<int WAVES, bool TILED> static hipError_t launch_gemv_t(const uint8_t* W
 	const size_t shmem = static_cast<size_t>(K) + static_cast<size_t>(K / QK) * 4 + WAVES * 64 * 4;
 	if (sums) {
 		gemv_kernel<WAVES, TILED, true><<<dim3(strips), dim3(WAVES * 64), shmem, s>>>(W, xq, y, sums, N, K);
-	} else {
-		gemv_kernel<WAVES, TILED, false><<<dim3(strips), dim3(WAVES * 64), shmem, s>>>(W, xq, y, sums, N, K);
+		return hipGetLastError();
 	}
-	return hipGetLastError();
+	return launch_kernel(KIND_GEMV, gemv_kernel<WAVES, TILED, false>, dim3(strips), dim3(WAVES * 64), shmem, s, W, xq, y, sums, N, K);
 }
 
 hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* sums, int64_t N, int64_t K, bool tiled, hipStream_t s) {

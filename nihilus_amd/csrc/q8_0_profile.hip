@@ -1,0 +1,169 @@
+// Opt-in per-kernel timing and the native batch runner.
+//
+// Timing: while it is on for one kernel kind, each launch of that kind carries a start/stop event pair in its
+// dispatch packet; nh_profile_end sums the elapsed times.  This measures the kernel alone (no launch gap), on the
+// stream it runs on, inside the caller's own timed loop.  Off by default: a plain launch costs one branch.
+//
+// Batch runner: a list of mul_mat operations enqueued from native code in one call, so a decode step's
+// launches (7 projections x 32 layers + lm_head at LLaMA-3-8B) are not paced by the caller's language runtime.
+#include "../../include/nihilus_amd/q8_0_abi.h"
+#include "q8_0_device.h"
+
+#include <mutex>
+#include <vector>
+
+namespace nh {
+
+namespace {
+	struct timer_state {
+		std::mutex lock;
+		int kind = -1; // kind being timed, -1 = off
+		std::vector<hipEvent_t> events; // 2 per launch
+		size_t used = 0; // events handed out
+	};
+	timer_state& timer() {
+		static timer_state t;
+		return t;
+	}
+} // namespace
+
+bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop) {
+	timer_state& t = timer();
+	if (t.kind != kind) { // unsynchronised fast path: timing is switched only while no launch is in flight
+		return false;
+	}
+	std::lock_guard<std::mutex> g(t.lock);
+	if (t.kind != kind || t.used + 2 > t.events.size()) {
+		return false;
+	}
+	*start = t.events[t.used];
+	*stop  = t.events[t.used + 1];
+	t.used += 2;
+	return true;
+}
+
+} // namespace nh
+
+extern "C" {
+
+int nh_profile_begin(int kernel_kind, int64_t max_launches) {
+	if (kernel_kind < 0 || kernel_kind >= nh::KIND_COUNT || max_launches <= 0 || max_launches > (1 << 20)) {
+		return NH_ERR_ARGUMENT;
+	}
+	nh::timer_state& t = nh::timer();
+	std::lock_guard<std::mutex> g(t.lock);
+	if (t.kind != -1) {
+		return NH_ERR_ARGUMENT; // already timing
+	}
+	t.events.resize(static_cast<size_t>(max_launches) * 2);
+	for (size_t i = 0; i < t.events.size(); ++i) {
+		const hipError_t e = hipEventCreate(&t.events[i]);
+		if (e != hipSuccess) {
+			for (size_t j = 0; j < i; ++j) {
+				(void)hipEventDestroy(t.events[j]);
+			}
+			t.events.clear();
+			return static_cast<int>(e);
+		}
+	}
+	t.used = 0;
+	t.kind = kernel_kind;
+	return NH_OK;
+}
+
+int nh_profile_end(double* host_total_ms, int64_t* host_launches, double* host_min_ms, double* host_max_ms) {
+	nh::timer_state& t = nh::timer();
+	std::lock_guard<std::mutex> g(t.lock);
+	if (t.kind == -1) {
+		return NH_ERR_ARGUMENT;
+	}
+	t.kind		 = -1;
+	int rc		 = NH_OK;
+	double total = 0.0, mn = 0.0, mx = 0.0;
+	int64_t n	 = 0;
+	for (size_t i = 0; i + 1 < t.used; i += 2) {
+		hipError_t e = hipEventSynchronize(t.events[i + 1]);
+		float ms	 = 0.0f;
+		if (e == hipSuccess) {
+			e = hipEventElapsedTime(&ms, t.events[i], t.events[i + 1]);
+		}
+		if (e != hipSuccess) {
+			rc = static_cast<int>(e);
+			break;
+		}
+		total += ms;
+		mn = (n == 0 || ms < mn) ? ms : mn;
+		mx = (n == 0 || ms > mx) ? ms : mx;
+		++n;
+	}
+	for (hipEvent_t ev : t.events) {
+		(void)hipEventDestroy(ev);
+	}
+	t.events.clear();
+	t.used = 0;
+	if (host_total_ms) {
+		*host_total_ms = total;
+	}
+	if (host_launches) {
+		*host_launches = n;
+	}
+	if (host_min_ms) {
+		*host_min_ms = mn;
+	}
+	if (host_max_ms) {
+		*host_max_ms = mx;
+	}
+	return rc;
+}
+
+int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, void* workspace, int64_t workspace_bytes, void* stream) {
+	if (count < 0) {
+		return NH_ERR_SHAPE;
+	}
+	if (count == 0) {
+		return NH_OK;
+	}
+	if (!host_ops) {
+		return NH_ERR_NULL_POINTER;
+	}
+	// validate everything before the first launch, so a bad entry cannot leave half a step enqueued
+	for (int64_t i = 0; i < count; ++i) {
+		const nh_q8_0_mul_mat_op& op = host_ops[i];
+		if (op.M < 0 || op.N < 0 || op.K < 0 || op.K % nh::GROUP_K != 0) {
+			return NH_ERR_SHAPE;
+		}
+		const int64_t need = nh_q8_0_mul_mat_workspace_bytes(op.M, op.K);
+		if (need < 0 || need > workspace_bytes) {
+			return NH_ERR_ARGUMENT;
+		}
+		if (op.M > 0 && op.N > 0 && (!op.W_tiled || !op.x || !op.y)) {
+			return NH_ERR_NULL_POINTER;
+		}
+	}
+	const float* quantized_x = nullptr; // activation currently held in the workspace
+	int64_t quantized_m = -1, quantized_k = -1;
+	for (int64_t i = 0; i < count; ++i) {
+		const nh_q8_0_mul_mat_op& op = host_ops[i];
+		if (op.M == 0 || op.N == 0) {
+			continue;
+		}
+		int rc				= NH_OK;
+		const bool reuse = op.reuse_quantized_x && quantized_x == op.x && quantized_m == op.M && quantized_k == op.K;
+		if (!reuse) {
+			rc = (op.M == 1) ? nh_q8_0_quantize(op.x, workspace, 1, op.K, stream) : nh_q8_0_quantize_tiled(op.x, workspace, op.M, op.K, stream);
+			if (rc != NH_OK) {
+				return rc;
+			}
+			quantized_x = op.x;
+			quantized_m = op.M;
+			quantized_k = op.K;
+		}
+		rc = (op.M == 1) ? nh_q8_0_gemv_tiled(op.W_tiled, workspace, op.y, op.N, op.K, stream) : nh_q8_0_gemm_tiled(op.W_tiled, workspace, op.y, op.M, op.N, op.K, stream);
+		if (rc != NH_OK) {
+			return rc;
+		}
+	}
+	return NH_OK;
+}
+
+} // extern "C"

@@ -36,8 +36,11 @@ template<bool TILED> __global__ __launch_bounds__(256) void quantize_kernel(cons
 	const uint16_t dh = float_to_half_bits(d);
 
 	auto q8 = [id](float f) -> uint32_t {
-		int q = static_cast<int>(rintf(__fmul_rn(f, id))); // v_rndne_f32: ties to even
-		q	  = max(-128, min(127, q)); // the reference's saturating packs; never active for finite input
+		const float r = rintf(__fmul_rn(f, id)); // v_rndne_f32: ties to even
+		// x86 cvtps_epi32 yields 0x80000000 for NaN and out-of-range values, which the reference's saturating packs
+		// turn into -128.  Reachable only when 127/amax overflows to inf (amax below ~3.7e-37): inf, and 0*inf = NaN.
+		int q = (fabsf(r) < 2147483648.0f) ? static_cast<int>(r) : INT32_MIN;
+		q	  = max(-128, min(127, q));
 		return static_cast<uint32_t>(q) & 0xFFu;
 	};
 	const uint32_t packed = q8(v.x) | (q8(v.y) << 8) | (q8(v.z) << 16) | (q8(v.w) << 24);
@@ -74,12 +77,11 @@ hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool
 		return hipSuccess;
 	}
 	const int64_t grid = (threads + 255) / 256;
+	const dim3 g(static_cast<unsigned>(grid)), b(256);
 	if (tiled) {
-		quantize_kernel<true><<<dim3(static_cast<unsigned>(grid)), dim3(256), 0, s>>>(x, static_cast<uint8_t*>(out), M, rows_out, K);
-	} else {
-		quantize_kernel<false><<<dim3(static_cast<unsigned>(grid)), dim3(256), 0, s>>>(x, static_cast<uint8_t*>(out), M, rows_out, K);
+		return launch_kernel(KIND_QUANTIZE, quantize_kernel<true>, g, b, 0, s, x, static_cast<uint8_t*>(out), M, rows_out, K);
 	}
-	return hipGetLastError();
+	return launch_kernel(KIND_QUANTIZE, quantize_kernel<false>, g, b, 0, s, x, static_cast<uint8_t*>(out), M, rows_out, K);
 }
 
 } // namespace nh

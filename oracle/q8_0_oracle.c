@@ -159,7 +159,7 @@ void nho_dequantize_row_q8_0(const void* vx, float* y, int64_t k) {
  *   d     = amax / 127.f in fp32, stored as fp16 RNE                   (:4460-4461)
  *   id    = amax != 0 ? 127.f / amax : 0                               (:4462)
  *   q_i   = (int8) round_half_even(x_i * id), product rounded to fp32 first   (:4465-4478)
- *   packs are saturating (:4480-4482) -- cannot trigger for finite input since |x_i*id| <= 127.
+ *   packs are saturating (:4480-4482) -- for finite input |x_i*id| <= 127 unless 127/amax overflows (see below).
  *   nb = k / 32; a trailing partial block is ignored                   (:4440)                */
 void nho_quantize_row_q8_0(const float* x, void* vy, int64_t k) {
 	uint8_t* y		 = (uint8_t*)vy;
@@ -182,7 +182,10 @@ void nho_quantize_row_q8_0(const float* x, void* vy, int64_t k) {
 		for (int j = 0; j < NHO_QK; ++j) {
 			volatile float p = xb[j] * id; /* one fp32 rounding, never fused with anything */
 			float r			 = nearbyintf(p); /* default rounding mode: ties to even */
-			int32_t q		 = (int32_t)r;
+			/* cvtps_epi32 (:4475-4478) returns the "integer indefinite" 0x80000000 for NaN and for values outside
+			 * int32; that only happens when 127/amax overflows to inf (amax below ~3.7e-37): inf and 0*inf = NaN
+			 * then both saturate to -128 in the packs. */
+			int32_t q = (r >= -2147483648.0f && r < 2147483648.0f) ? (int32_t)r : INT32_MIN;
 			if (q > 127) {
 				q = 127;
 			}
