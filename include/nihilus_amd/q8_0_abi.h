@@ -144,9 +144,12 @@ int nh_profile_end(double* host_total_ms, int64_t* host_launches, double* host_m
 /* Parity instrumentation ------------------------------------------------------------------------ */
 
 /* Per-(m, n, block) int32 sums as the production kernels compute them (same device code path, results
- * diverted before scaling): sums[(m*N + n)*(K/32) + b].  path 0 = the GEMV kernel's v_dot4 path
- * (M must be 1), path 1 = the GEMM kernel's MFMA path.  Operands in the blocks layout. */
-int nh_q8_0_debug_block_sums(const void* W_blocks, const void* Aq_blocks, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream);
+ * diverted before scaling): sums[(m*N + n)*(K/32) + b].
+ *   path 0  mat-vec kernel on the blocks layout (v_dot4), M must be 1; W and Aq in the blocks layout
+ *   path 1  mat-mat kernel on the blocks layout (MFMA);             W and Aq in the blocks layout
+ *   path 2  streaming mat-vec kernel on the tiled layout, M must be 1; W tiled, Aq = one row of blocks
+ *   path 3  mat-mat kernel on the tiled layout (MFMA);               W and Aq tiled */
+int nh_q8_0_debug_block_sums(const void* W, const void* Aq, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream);
 
 /* Synthetic inputs (benchmark / test utility) --------------------------------------------------- */
 

@@ -313,20 +313,22 @@ int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, in
 	return nh_q8_0_gemm_tiled(W_tiled, workspace, y, M, N, K, stream);
 }
 
-int nh_q8_0_debug_block_sums(const void* W_blocks, const void* Aq_blocks, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream) {
-	NH_TRY(check_shape(M, N, K, false));
-	NH_REQUIRE(path == 0 || path == 1, NH_ERR_ARGUMENT);
-	NH_REQUIRE(path == 1 || M == 1, NH_ERR_ARGUMENT);
+int nh_q8_0_debug_block_sums(const void* W, const void* Aq, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream) {
+	NH_REQUIRE(path >= 0 && path <= 3, NH_ERR_ARGUMENT);
+	const bool tiled = path >= 2;
+	const bool mfma	 = (path & 1) != 0;
+	NH_TRY(check_shape(M, N, K, tiled));
+	NH_REQUIRE(mfma || M == 1, NH_ERR_ARGUMENT);
 	if (M == 0 || N == 0 || K == 0) {
 		return NH_OK;
 	}
-	NH_REQUIRE(W_blocks && Aq_blocks && sums, NH_ERR_NULL_POINTER);
-	NH_REQUIRE(aligned16(W_blocks) && aligned16(Aq_blocks) && aligned16(sums), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(W && Aq && sums, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(W) && aligned16(Aq) && aligned16(sums), NH_ERR_ALIGNMENT);
 	NH_TRY(require_device());
-	if (path == 0) {
-		return from_hip(nh::launch_gemv(W_blocks, Aq_blocks, nullptr, sums, N, K, false, as_stream(stream)));
+	if (!mfma) {
+		return from_hip(nh::launch_gemv(W, Aq, nullptr, sums, N, K, tiled, as_stream(stream)));
 	}
-	return from_hip(nh::launch_gemm(W_blocks, Aq_blocks, nullptr, sums, M, N, K, false, as_stream(stream)));
+	return from_hip(nh::launch_gemm(W, Aq, nullptr, sums, M, N, K, tiled, as_stream(stream)));
 }
 
 int nh_q8_0_fill_weight_blocks(void* blocks, uint64_t seed, int64_t first_block, int64_t n_blocks, void* stream) {

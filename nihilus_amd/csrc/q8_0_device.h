@@ -20,6 +20,7 @@ constexpr int MACRO_D_OFFSET = GROUP_BLOCKS * TILE_BYTES; // 4096
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
 
 // fp16 bits -> fp32, exact (v_cvt_f32_f16; fp16 subnormals are honoured: the kernel's float mode keeps them).
 __device__ __forceinline__ float half_bits_to_float(uint16_t h) {

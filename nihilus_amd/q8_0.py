@@ -107,10 +107,10 @@ def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: t
     return y
 
 
-def debug_block_sums(w_blocks: torch.Tensor, aq_blocks: torch.Tensor, m: int, n: int, k: int, path: int) -> torch.Tensor:
-    """int32 [m, n, k/32] block sums from the GEMV (path 0) or MFMA (path 1) kernel."""
-    sums = torch.empty((m, n, k // QK), dtype=torch.int32, device=w_blocks.device)
-    _lib.check("nh_q8_0_debug_block_sums", _lib.lib().nh_q8_0_debug_block_sums(w_blocks.data_ptr(), aq_blocks.data_ptr(), sums.data_ptr(), m, n, k, path, _stream()))
+def debug_block_sums(w: torch.Tensor, aq: torch.Tensor, m: int, n: int, k: int, path: int) -> torch.Tensor:
+    """int32 [m, n, k/32] block sums: path 0/1 = mat-vec / MFMA kernel on blocks, 2/3 = the same on the tiled layout."""
+    sums = torch.full((m, n, k // QK), -(2**31), dtype=torch.int32, device=w.device)
+    _lib.check("nh_q8_0_debug_block_sums", _lib.lib().nh_q8_0_debug_block_sums(w.data_ptr(), aq.data_ptr(), sums.data_ptr(), m, n, k, path, _stream()))
     return sums
 
 

@@ -34,6 +34,10 @@ def test_gemm_block_sums_exact(q8, oracle, m, n, k):
     got = to_host(q8.debug_block_sums(to_dev(w), to_dev(aq.reshape(-1)), m, n, k, path=1))
     for i in range(m):
         assert np.array_equal(got[i], oracle.block_sums_gemv(w, aq[i], n, k)), i
+    if k % 128 == 0:
+        wd, aqd = to_dev(w), to_dev(aq.reshape(-1))
+        got_t = to_host(q8.debug_block_sums(q8.tile(wd, n, k), q8.tile(aqd, m, k), m, n, k, path=3))
+        assert np.array_equal(got_t, got)
 
 
 def test_gemm_equals_gemvs(q8, oracle):

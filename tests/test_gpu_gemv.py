@@ -10,7 +10,7 @@ from helpers import REL_L2_TOL, random_blocks, rel_l2, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336), (1024, 4096), (96, 512), (33, 128), (1, 128), (31, 256), (257, 8192)]
+SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336), (1024, 4096), (96, 512), (33, 128), (1, 128), (31, 256), (257, 8192), (8192, 28672), (1024, 8192), (100, 40960)]
 
 
 def _inputs(oracle, n, k, seed):
@@ -28,18 +28,21 @@ def test_gemv_tiled_and_blocks(q8, oracle, n, k):
     y_tiled = to_host(q8.gemv(q8.tile(wd, n, k), xqd, n, k, tiled=True))
     assert rel_l2(y_blocks, want) <= REL_L2_TOL
     assert rel_l2(y_tiled, want) <= REL_L2_TOL
-    # both layouts hold the same values and the kernel sums them in the same order
-    assert np.array_equal(y_blocks, y_tiled)
+    # the two kernels sum in different orders; they agree far inside the contract
+    assert rel_l2(y_blocks, y_tiled) < 2e-6
     # far tighter than the contract in practice
     assert rel_l2(y_tiled, oracle.gemv_f64(w, xq, n, k)) < 5e-6
 
 
-@pytest.mark.parametrize("n,k", [(4096, 4096), (96, 512), (33, 160), (5, 32)])
+@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (96, 512), (33, 160), (5, 32), (64, 28672), (40, 128)])
 def test_gemv_block_sums_exact(q8, oracle, n, k):
     w, x, xq = _inputs(oracle, n, k, seed=5)
     want = oracle.block_sums_gemv(w, xq, n, k)
     got = to_host(q8.debug_block_sums(to_dev(w), to_dev(xq), 1, n, k, path=0))[0]
     assert np.array_equal(got, want)
+    if k % 128 == 0:  # the streaming kernel on the tiled layout
+        got = to_host(q8.debug_block_sums(q8.tile(to_dev(w), n, k), to_dev(xq), 1, n, k, path=2))[0]
+        assert np.array_equal(got, want)
 
 
 def test_gemv_ragged_k_blocks_layout(q8, oracle):
@@ -86,3 +89,15 @@ def test_gemv_errors(q8):
     assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 0, None) == 0  # empty dot product
     torch.cuda.synchronize()
     assert bool((y == 0.0).all())
+
+
+def test_gemv_split_k_is_deterministic_and_reusable(q8, oracle):
+    # few rows, long K: K is split over several workgroups whose partial sums are added by the last arriver in a
+    # fixed order -- repeated launches must give identical bits, and the arrival counters must be left ready
+    n, k = 4096, 14336
+    w, x, xq = _inputs(oracle, n, k, seed=77)
+    wt, xqd = q8.tile(to_dev(w), n, k), to_dev(xq)
+    first = to_host(q8.gemv(wt, xqd, n, k, tiled=True))
+    for _ in range(20):
+        assert np.array_equal(to_host(q8.gemv(wt, xqd, n, k, tiled=True)), first)
+    assert rel_l2(first, oracle.gemv(w, xq, n, k)) <= REL_L2_TOL
