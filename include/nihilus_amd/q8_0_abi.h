@@ -99,6 +99,13 @@ int nh_q8_0_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, voi
 int nh_q8_0_gemv(const void* W_blocks, const void* xq_blocks, float* y, int64_t N, int64_t K, void* stream);
 int nh_q8_0_gemv_tiled(const void* W_tiled, const void* xq_blocks, float* y, int64_t N, int64_t K, void* stream);
 
+/* Fused decode step: y = W . quantize(x) with the quantize done inside the mat-vec kernel (no separate launch, the
+ * quantized row never travels through memory).  x: fp32 [K].  Same values as nh_q8_0_quantize + nh_q8_0_gemv_tiled. */
+int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream);
+/* The same for up to 3 weight matrices that share K and x (q/k/v, gate/up: infra/core_traits.hpp:575-594, :976-986)
+ * as ONE launch: y[i] = W_tiled[i] . quantize(x), i < count.  host_* arrays are host memory, read before return. */
+int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream);
+
 /* Mat-mat (prefill, prompt_eval_time) ----------------------------------------------------------- */
 
 /* C[m*N + n] (n fastest, ggml's dst[ir1*nr0 + ir0], cpu/avx_2.hpp:4934) = the same dot for activation
@@ -150,6 +157,10 @@ int nh_profile_end(double* host_total_ms, int64_t* host_launches, double* host_m
  *   path 2  streaming mat-vec kernel on the tiled layout, M must be 1; W tiled, Aq = one row of blocks
  *   path 3  mat-mat kernel on the tiled layout (MFMA);               W and Aq tiled */
 int nh_q8_0_debug_block_sums(const void* W, const void* Aq, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream);
+
+/* What the fused mat-vec stages for x: runs the fused kernel's own quantize-and-stage code on fp32 x [K] and writes
+ * the staged row back as K/32 packed blocks, to be compared byte for byte with nh_q8_0_quantize. K % 128 == 0. */
+int nh_q8_0_debug_fused_quantize(const float* x, void* xq_blocks_out, int64_t K, void* stream);
 
 /* Synthetic inputs (benchmark / test utility) --------------------------------------------------- */
 

@@ -10,7 +10,8 @@ namespace {
 
 constexpr int64_t MAX_ROWS = int64_t{ 1 } << 30; // row and strip indices are 32-bit inside the kernels
 constexpr int64_t MAX_BLOCKS = int64_t{ 1 } << 35; // blocks per matrix the element-wise kernels can index
-constexpr int64_t MAX_K	   = 49152; // the mat-vec keeps the whole activation row (K + K/8 bytes) in 64 KiB of LDS
+constexpr int64_t MAX_K	   = int64_t{ 1 } << 24; // block and group indices along K are 32-bit
+constexpr int64_t MAX_K_BLOCKS_GEMV = 49152; // the blocks-layout mat-vec keeps the whole activation row (K + K/8 bytes) in 64 KiB of LDS
 
 inline bool aligned16(const void* p) {
 	return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
@@ -239,6 +240,7 @@ int nh_q8_0_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, voi
 
 static int gemv_common(const void* W, const void* xq, float* y, int64_t N, int64_t K, bool tiled, void* stream) {
 	NH_TRY(check_shape(N, 0, K, tiled));
+	NH_REQUIRE(tiled || K <= MAX_K_BLOCKS_GEMV, NH_ERR_TOO_LARGE);
 	if (N == 0) {
 		return NH_OK;
 	}
@@ -258,6 +260,55 @@ int nh_q8_0_gemv(const void* W_blocks, const void* xq_blocks, float* y, int64_t 
 
 int nh_q8_0_gemv_tiled(const void* W_tiled, const void* xq_blocks, float* y, int64_t N, int64_t K, void* stream) {
 	return gemv_common(W_tiled, xq_blocks, y, N, K, true, stream);
+}
+
+int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream) {
+	NH_REQUIRE(count >= 0 && count <= nh::GEMV_MAX_SEGMENTS, NH_ERR_ARGUMENT);
+	if (count == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(host_W_tiled && host_y && host_N, NH_ERR_NULL_POINTER);
+	int64_t rows = 0;
+	for (int64_t i = 0; i < count; ++i) {
+		NH_TRY(check_shape(host_N[i], 0, K, true));
+		rows += host_N[i];
+	}
+	NH_REQUIRE(rows <= MAX_ROWS, NH_ERR_TOO_LARGE);
+	if (rows == 0) {
+		return NH_OK;
+	}
+	for (int64_t i = 0; i < count; ++i) {
+		if (host_N[i] == 0) {
+			continue;
+		}
+		NH_REQUIRE(host_y[i], NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(host_y[i]), NH_ERR_ALIGNMENT);
+		if (K > 0) {
+			NH_REQUIRE(host_W_tiled[i], NH_ERR_NULL_POINTER);
+			NH_REQUIRE(aligned16(host_W_tiled[i]), NH_ERR_ALIGNMENT);
+		}
+	}
+	if (K > 0) {
+		NH_REQUIRE(x, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(x), NH_ERR_ALIGNMENT);
+	}
+	NH_TRY(require_device());
+	return from_hip(nh::launch_gemv_tiled_multi(host_W_tiled, host_y, host_N, static_cast<int>(count), x, true, K, as_stream(stream)));
+}
+
+int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream) {
+	return nh_q8_0_gemv_tiled_multi_f32(&W_tiled, &y, &N, 1, x, K, stream);
+}
+
+int nh_q8_0_debug_fused_quantize(const float* x, void* xq_blocks_out, int64_t K, void* stream) {
+	NH_TRY(check_shape(1, 0, K, true));
+	if (K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(x && xq_blocks_out, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(x) && aligned16(xq_blocks_out), NH_ERR_ALIGNMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_gemv_dump_staged_x(x, xq_blocks_out, K, as_stream(stream)));
 }
 
 static int gemm_common(const void* W, const void* A, float* C, int64_t M, int64_t N, int64_t K, bool tiled, void* stream) {
@@ -306,8 +357,7 @@ int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, in
 		NH_REQUIRE(aligned16(workspace) && aligned16(x), NH_ERR_ALIGNMENT);
 	}
 	if (M == 1) {
-		NH_TRY(nh_q8_0_quantize(x, workspace, 1, K, stream));
-		return nh_q8_0_gemv_tiled(W_tiled, workspace, y, N, K, stream);
+		return nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream); // quantize fused into the mat-vec: the workspace stays unused
 	}
 	NH_TRY(nh_q8_0_quantize_tiled(x, workspace, M, K, stream));
 	return nh_q8_0_gemm_tiled(W_tiled, workspace, y, M, N, K, stream);
@@ -319,6 +369,7 @@ int nh_q8_0_debug_block_sums(const void* W, const void* Aq, int32_t* sums, int64
 	const bool mfma	 = (path & 1) != 0;
 	NH_TRY(check_shape(M, N, K, tiled));
 	NH_REQUIRE(mfma || M == 1, NH_ERR_ARGUMENT);
+	NH_REQUIRE(mfma || tiled || K <= MAX_K_BLOCKS_GEMV, NH_ERR_TOO_LARGE);
 	if (M == 0 || N == 0 || K == 0) {
 		return NH_OK;
 	}

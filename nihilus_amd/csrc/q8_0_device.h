@@ -50,6 +50,29 @@ __device__ __forceinline__ uint16_t load_u16(const uint8_t* p) {
 	return *reinterpret_cast<const uint16_t*>(p);
 }
 
+// One lane's share of quantize_row_q8_0 (reference cpu/avx_2.hpp:4439-4489): eight consecutive lanes hold one
+// 32-value block as eight float4.  Returns this lane's four quants packed little-endian; *dh = fp16 bits of d.
+//   amax = max|x_i|; d = fp16_rne(amax / 127.f); id = amax != 0 ? 127.f / amax : 0; q_i = int8(rne(fl32(x_i * id)))
+// Divide, multiply and rounding are separate correctly rounded fp32 operations; all eight lanes must be active.
+__device__ __forceinline__ uint32_t quantize_block_lane(float4 v, uint16_t* dh) {
+	float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+	amax	   = fmaxf(amax, __shfl_xor(amax, 1));
+	amax	   = fmaxf(amax, __shfl_xor(amax, 2));
+	amax	   = fmaxf(amax, __shfl_xor(amax, 4));
+	const float d  = __fdiv_rn(amax, 127.0f);
+	const float id = (amax != 0.0f) ? __fdiv_rn(127.0f, amax) : 0.0f;
+	*dh			   = float_to_half_bits(d);
+	auto q8		   = [id](float f) -> uint32_t {
+		   const float r = rintf(__fmul_rn(f, id)); // v_rndne_f32: ties to even
+		   // x86 cvtps_epi32 yields 0x80000000 for NaN and out-of-range values, which the reference's saturating packs
+		   // turn into -128.  Reachable only when 127/amax overflows to inf (amax below ~3.7e-37): inf, and 0*inf = NaN.
+		   int q = (fabsf(r) < 2147483648.0f) ? static_cast<int>(r) : INT32_MIN;
+		   q	 = max(-128, min(127, q));
+		   return static_cast<uint32_t>(q) & 0xFFu;
+	};
+	return q8(v.x) | (q8(v.y) << 8) | (q8(v.z) << 16) | (q8(v.w) << 24);
+}
+
 // Byte offset of macro-tile (strip, group) in a tiled matrix with `groups` = K/128 groups per strip.
 __device__ __host__ __forceinline__ int64_t macro_offset(int64_t strip, int64_t group, int64_t groups) {
 	return (strip * groups + group) * MACRO_BYTES;
@@ -84,6 +107,13 @@ hipError_t launch_fill_weights(void* blocks, uint64_t seed, int64_t first_block,
 hipError_t launch_fill_activations(float* x, uint64_t seed, int64_t count, hipStream_t s);
 // sums == nullptr: production; otherwise the same kernel diverts the per-block int32 sums to `sums` and leaves y alone.
 hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* sums, int64_t N, int64_t K, bool tiled, hipStream_t s);
+// Streaming mat-vec on tiled weights for up to GEMV_MAX_SEGMENTS matrices that share K and the activation row:
+// one launch computes y[i] = W[i] . x for all of them.  x is either one row of packed blocks (x_is_f32 = false)
+// or the fp32 activations themselves, quantized inside the kernel (x_is_f32 = true).
+constexpr int GEMV_MAX_SEGMENTS = 3;
+hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s);
+// Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
+hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s);
 hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s);
 
 } // namespace nh

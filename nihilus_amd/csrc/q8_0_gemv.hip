@@ -2,27 +2,23 @@
 //
 // Computes vec_dot_q8_0_q8_0 (reference cpu/avx_2.hpp:4534-4747) for every weight row:
 //   y[n] = sum_b f32(dW[n][b]) * f32(dx[b]) * (sum_j W.qs[n][b][j] * x.qs[b][j])
-// with exact int32 block sums (v_dot4_i32_i8) and fp32 scale-and-accumulate.
+// with exact int32 block sums (v_dot4_i32_i8) and fp32 scale-and-accumulate.  HBM-bound: 34 bytes of weight
+// per 32 multiply-adds, each read exactly once.
 //
-// HBM-bound: 34 bytes of weight per 32 multiply-adds, read exactly once.
-//   * one workgroup per 32-row strip; its waves split the strip's K range into 128-quant groups and
-//     walk them interleaved, so the workgroup streams one contiguous span of the tiled matrix;
-//   * per group a lane issues four 16-byte loads (one KiB per wavefront each, fully coalesced in the
-//     tiled layout) plus one 8-byte load of its row's four block scales;
-//   * the activation row is staged once in LDS (quants as 16-byte chunks, scales as fp32); each lane
-//     reads its 16-byte chunk as a two-address broadcast;
-//   * lane l accumulates row (l%32), quants 16*(l/32).. of every block: no cross-lane reduction in the
-//     loop; halves and waves are combined once through LDS, in a fixed order (run-to-run bit-stable).
-// The same kernel reads the reference's packed 34-byte blocks directly (TILED = false) with unaligned
-// 16-byte loads; that is the drop-in-on-raw-bytes form and the parity twin of the tiled one.
+// Two kernels:
+//   gemv_blocks_kernel  reads the reference's packed 34-byte blocks as they are (unaligned 16-byte loads):
+//                       the drop-in-on-raw-bytes form, and the parity twin of the streaming kernel;
+//   gemv_tiled_kernel   the streaming kernel on the tiled layout -- the one the decode path runs.
+// In both, lane l accumulates row (l % 32), quants 16*(l/32).. of every block, so the loop needs no cross-lane
+// reduction; halves and waves are combined once through LDS in a fixed order (run-to-run bit-stable).
 #include "q8_0_device.h"
 
 #include <mutex>
 
 namespace nh {
 
-template<int WAVES, bool TILED, bool DUMP>
-__global__ __launch_bounds__(WAVES * 64) void gemv_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq, float* __restrict__ y, int32_t* __restrict__ sums, int N, int K) {
+template<int WAVES, bool DUMP>
+__global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq, float* __restrict__ y, int32_t* __restrict__ sums, int N, int K) {
 	extern __shared__ __align__(16) uint8_t smem[];
 	const int nb	 = K / QK;
 	const int groups = (nb + GROUP_BLOCKS - 1) / GROUP_BLOCKS;
@@ -53,38 +49,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(const uint8_t* __restr
 	__syncthreads();
 
 	const int64_t row_bytes = static_cast<int64_t>(nb) * BLOCK_BYTES;
-	const uint8_t* w_row	= W + row_c * row_bytes; // blocks layout
-	const uint8_t* w_strip	= W + macro_offset(strip, 0, groups); // tiled layout
+	const uint8_t* w_row	= W + row_c * row_bytes;
 
 	float acc = 0.0f;
 #pragma unroll 2
 	for (int g = wave; g < groups; g += WAVES) {
 		v4i q[GROUP_BLOCKS];
 		float dw[GROUP_BLOCKS];
-		if constexpr (TILED) {
-			const uint8_t* macro = w_strip + static_cast<int64_t>(g) * MACRO_BYTES;
 #pragma unroll
-			for (int t = 0; t < GROUP_BLOCKS; ++t) {
-				q[t] = *reinterpret_cast<const v4i*>(macro + t * TILE_BYTES + 16 * lane);
-			}
-			const uint2 dd = *reinterpret_cast<const uint2*>(macro + MACRO_D_OFFSET + 8 * r);
-			dw[0]		   = half_bits_to_float(static_cast<uint16_t>(dd.x & 0xFFFFu));
-			dw[1]		   = half_bits_to_float(static_cast<uint16_t>(dd.x >> 16));
-			dw[2]		   = half_bits_to_float(static_cast<uint16_t>(dd.y & 0xFFFFu));
-			dw[3]		   = half_bits_to_float(static_cast<uint16_t>(dd.y >> 16));
-		} else {
-#pragma unroll
-			for (int t = 0; t < GROUP_BLOCKS; ++t) {
-				const int b		   = min(g * GROUP_BLOCKS + t, nb - 1); // ragged last group: clamped, masked below
-				const uint8_t* blk = w_row + static_cast<int64_t>(b) * BLOCK_BYTES;
-				q[t]			   = load16_unaligned(blk + 2 + 16 * half);
-				dw[t]			   = half_bits_to_float(load_u16(blk));
-			}
+		for (int t = 0; t < GROUP_BLOCKS; ++t) {
+			const int b		   = min(g * GROUP_BLOCKS + t, nb - 1); // ragged last group: clamped, masked below
+			const uint8_t* blk = w_row + static_cast<int64_t>(b) * BLOCK_BYTES;
+			q[t]			   = load16_unaligned(blk + 2 + 16 * half);
+			dw[t]			   = half_bits_to_float(load_u16(blk));
 		}
 #pragma unroll
 		for (int t = 0; t < GROUP_BLOCKS; ++t) {
 			const int b = g * GROUP_BLOCKS + t;
-			if (TILED || b < nb) {
+			if (b < nb) {
 				const v4i xv = *reinterpret_cast<const v4i*>(xs_q + b * QK + 16 * half);
 				const int s	 = dot16(q[t], xv);
 				if constexpr (DUMP) {
@@ -123,82 +105,125 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(const uint8_t* __restr
 //   * sixteen waves per workgroup, one workgroup per (32-row strip, K split); every wave owns at most TILES
 //     128-quant groups and issues ALL of its weight loads (TILES x (4 x 16 B + 8 B) per lane, non-temporal)
 //     before it waits for anything: no loop, no workgroup barrier in front of the loads;
-//   * its slice of the activation row is staged wave-locally: the loads for it go out first, are re-aligned
-//     from the packed 34-byte blocks into LDS as the weight loads fly, and are read back as 16-byte
-//     two-address broadcasts (only the wave's own lgkm counter is waited on, never a barrier);
+//   * its slice of the activation row is staged wave-locally while the weight loads fly, either re-aligned
+//     from packed 34-byte blocks (XF32 = false) or quantized on the spot from the fp32 activations with the
+//     very arithmetic of the stand-alone quantize kernel (XF32 = true: no separate quantize launch, no
+//     round trip of the quantized row through memory); it is read back as 16-byte two-address broadcasts
+//     (only the wave's own LDS counter is waited on, never a barrier);
 //   * one LDS reduction per workgroup; when K is split over several workgroups (few rows, long K) each writes
 //     32 partial sums and the last to arrive adds them in split order -- fixed order, so results do not
-//     depend on arrival order.
+//     depend on arrival order;
+//   * up to three weight matrices that share K and the activation row (q/k/v, gate/up) run as one launch:
+//     a bigger launch amortises the ramp-up and the tail.
 constexpr int GEMV_WAVES = 16;
 
-template<int TILES, bool DUMP>
-__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ xq, float* __restrict__ y, int32_t* __restrict__ sums,
-	float* __restrict__ partials, unsigned* __restrict__ counters, int N, int groups, int splits) {
-	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K]; // this wave's activation quants, block jj at 32*jj
-	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
-	__shared__ float red[GEMV_WAVES][64];
-	__shared__ int last_flag;
+struct gemv_segments {
+	const uint8_t* W[GEMV_MAX_SEGMENTS];
+	float* y[GEMV_MAX_SEGMENTS];
+	int rows[GEMV_MAX_SEGMENTS];
+	int strip_end[GEMV_MAX_SEGMENTS]; // running total of strips
+};
 
-	const int tid	= threadIdx.x;
-	const int lane	= tid & 63;
-	const int wave	= tid >> 6;
-	const int strip = blockIdx.x / splits;
-	const int split = blockIdx.x - strip * splits;
-	const int slots = splits * GEMV_WAVES;
-	const int slot	= split * GEMV_WAVES + wave;
-	const int g0	= static_cast<int>((static_cast<int64_t>(groups) * slot) / slots);
-	const int g1	= static_cast<int>((static_cast<int64_t>(groups) * (slot + 1)) / slots);
-	const int cnt	= g1 - g0; // <= TILES (the host picks splits so)
-	const int r		= lane & 31;
-	const int half	= lane >> 5;
+enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
 
-	// ---- 1. activation slice: raw dwords of blocks [4*g0, 4*g1), 34 dwords per group, issued first ----
-	const uint32_t* x_raw = reinterpret_cast<const uint32_t*>(xq + static_cast<int64_t>(g0) * (GROUP_BLOCKS * BLOCK_BYTES));
-	constexpr int X_DWORDS = TILES * 34;
-	constexpr int X_LOADS  = (X_DWORDS + 63) / 64;
-	uint32_t xr[X_LOADS];
-#pragma unroll
-	for (int i = 0; i < X_LOADS; ++i) {
-		const int sidx = lane + 64 * i;
-		xr[i]		   = sidx < cnt * 34 ? x_raw[sidx] : 0u;
-	}
+// One chunk of a wave's K range: groups [gc, gc + cnt), cnt <= TILES, all wave-uniform (scalar registers).
+// xs_q / xs_d are this wave's private LDS slices.  Returns the lane's partial dot product over the chunk.
+template<int TILES, bool XF32, int DUMP>
+__device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
+	int groups, int lane, int row, int N, bool dump_this_strip) {
+	const int r	   = lane & 31;
+	const int half = lane >> 5;
 
-	// ---- 2. every weight byte this wave will ever need, in flight at once ----
-	v4i q[TILES][GROUP_BLOCKS];
-	v2u dd[TILES];
-	const uint8_t* macro0 = W + macro_offset(strip, g0, groups);
+	// ---- 1. activation slice loads, issued first ----
+	constexpr int XQ_LOADS = (TILES * 34 + 63) / 64; // raw dwords of blocks [4*gc, 4*(gc+cnt)): 34 dwords per group
+	constexpr int XF_LOADS = (TILES * 32 + 63) / 64; // float4 per lane: 128 floats per group = 32 float4
+	uint32_t xr[XQ_LOADS];
+	float4 xf[XF_LOADS];
+	if constexpr (XF32) {
+		const float4* x4 = reinterpret_cast<const float4*>(static_cast<const float*>(xin) + static_cast<int64_t>(gc) * GROUP_K);
 #pragma unroll
-	for (int t = 0; t < TILES; ++t) {
-		if (t < cnt) {
-			const uint8_t* macro = macro0 + static_cast<int64_t>(t) * MACRO_BYTES;
+		for (int i = 0; i < XF_LOADS; ++i) {
+			const int v = lane + 64 * i; // float4 index in the slice; block = v / 8
+			xf[i]		= v < cnt * 32 ? x4[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+		}
+	} else {
+		const uint32_t* x_raw = reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(xin) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * BLOCK_BYTES));
 #pragma unroll
-			for (int j = 0; j < GROUP_BLOCKS; ++j) {
-				q[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
-			}
-			dd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+		for (int i = 0; i < XQ_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			xr[i]		= v < cnt * 34 ? x_raw[v] : 0u;
 		}
 	}
 
-	// ---- 3. re-align the activation slice into LDS: half-word hw of the raw stream is scale (hw%17 == 0) or a quant pair ----
+	// ---- 2. every weight byte of the chunk, in flight at once ----
+	v4i q[TILES][GROUP_BLOCKS];
+	v2u dd[TILES];
+	if constexpr (DUMP != DUMP_X) {
+		const uint8_t* macro0 = w_strip + static_cast<int64_t>(gc) * MACRO_BYTES;
 #pragma unroll
-	for (int i = 0; i < X_LOADS; ++i) {
-		const int sidx = lane + 64 * i;
-		if (sidx < cnt * 34) {
+		for (int t = 0; t < TILES; ++t) {
+			if (t < cnt) {
+				const uint8_t* macro = macro0 + t * MACRO_BYTES;
 #pragma unroll
-			for (int h = 0; h < 2; ++h) {
-				const int hw	   = 2 * sidx + h;
-				const int jj	   = hw / 17;
-				const int o		   = hw - 17 * jj;
-				const uint16_t val = static_cast<uint16_t>(h ? (xr[i] >> 16) : (xr[i] & 0xFFFFu));
-				if (o == 0) {
-					xs_d[wave][jj] = half_bits_to_float(val);
-				} else {
-					*reinterpret_cast<uint16_t*>(&xs_q[wave][jj * QK + 2 * (o - 1)]) = val;
+				for (int j = 0; j < GROUP_BLOCKS; ++j) {
+					q[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+				}
+				dd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+			}
+		}
+	}
+
+	// ---- 3. stage the activation slice in LDS: quants 16-byte aligned per half block, scales as fp32 ----
+	if constexpr (XF32) {
+#pragma unroll
+		for (int i = 0; i < XF_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			uint16_t dh;
+			const uint32_t packed = quantize_block_lane(xf[i], &dh); // all lanes take part; lanes past the slice hold zeros
+			if (v < cnt * 32) {
+				*reinterpret_cast<uint32_t*>(xs_q + 4 * v) = packed; // block v/8 at 32*(v/8), dword v%8
+				if ((v & 7) == 0) {
+					xs_d[v >> 3] = half_bits_to_float(dh); // the fp16-rounded scale, exactly what a stored block would hold
+				}
+			}
+		}
+	} else {
+		// half-word hw of the raw stream is a scale (hw % 17 == 0) or a quant pair
+#pragma unroll
+		for (int i = 0; i < XQ_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			if (v < cnt * 34) {
+#pragma unroll
+				for (int h = 0; h < 2; ++h) {
+					const int hw	   = 2 * v + h;
+					const int jj	   = hw / 17;
+					const int o		   = hw - 17 * jj;
+					const uint16_t val = static_cast<uint16_t>(h ? (xr[i] >> 16) : (xr[i] & 0xFFFFu));
+					if (o == 0) {
+						xs_d[jj] = half_bits_to_float(val);
+					} else {
+						*reinterpret_cast<uint16_t*>(xs_q + jj * QK + 2 * (o - 1)) = val;
+					}
 				}
 			}
 		}
 	}
-	__builtin_amdgcn_wave_barrier(); // wave-local hand-off: same wave wrote and reads, the LDS counter wait orders it
+	__builtin_amdgcn_wave_barrier(); // wave-local hand-off: the same wave wrote and reads; the LDS counter wait orders it
+
+	if constexpr (DUMP == DUMP_X) {
+		// parity hook: what was staged, written back as packed blocks (the first strip of the launch covers all of K)
+		if (dump_this_strip) {
+			uint8_t* out = static_cast<uint8_t*>(dump) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * BLOCK_BYTES);
+			for (int jj = lane; jj < cnt * GROUP_BLOCKS; jj += 64) {
+				uint8_t* o						= out + jj * BLOCK_BYTES;
+				*reinterpret_cast<uint16_t*>(o) = float_to_half_bits(xs_d[jj]); // exact: the value came from fp16
+				for (int i = 0; i < 16; ++i) {
+					*reinterpret_cast<uint16_t*>(o + 2 + 2 * i) = *reinterpret_cast<const uint16_t*>(xs_q + jj * QK + 2 * i);
+				}
+			}
+		}
+		return 0.0f;
+	}
 
 	// ---- 4. dot products as the tiles land ----
 	float acc = 0.0f;
@@ -210,25 +235,61 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(const uint8
 #pragma unroll
 			for (int j = 0; j < GROUP_BLOCKS; ++j) {
 				const int jj = t * GROUP_BLOCKS + j;
-				const v4i xv = *reinterpret_cast<const v4i*>(&xs_q[wave][jj * QK + 16 * half]);
+				const v4i xv = *reinterpret_cast<const v4i*>(xs_q + jj * QK + 16 * half);
 				const int s	 = dot16(q[t][j], xv);
-				if constexpr (DUMP) {
+				if constexpr (DUMP == DUMP_SUMS) {
 					const int full = s + __shfl_xor(s, 32);
-					const int row  = strip * STRIP_ROWS + r;
 					if (half == 0 && row < N) {
-						sums[static_cast<int64_t>(row) * (groups * GROUP_BLOCKS) + (g0 * GROUP_BLOCKS + jj)] = full;
+						static_cast<int32_t*>(dump)[static_cast<int64_t>(row) * (groups * GROUP_BLOCKS) + (gc * GROUP_BLOCKS + jj)] = full;
 					}
 				} else {
-					acc = fmaf(static_cast<float>(s), dw[j] * xs_d[wave][jj], acc);
+					acc = fmaf(static_cast<float>(s), dw[j] * xs_d[jj], acc);
 				}
 			}
 		}
 	}
-	if constexpr (DUMP) {
+	return acc;
+}
+
+template<int TILES, bool XF32, int DUMP, bool LOOP>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, float* __restrict__ partials,
+	unsigned* __restrict__ counters, int groups, int split_shift, int groups_per_slot, int groups_rem) {
+	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K]; // each wave's activation quants, block jj at 32*jj
+	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
+	__shared__ float red[GEMV_WAVES][64];
+	__shared__ int last_flag;
+
+	const int tid	 = threadIdx.x;
+	const int lane	 = tid & 63;
+	const int wave	 = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform by construction: keep it (and all that follows from it) scalar
+	const int splits = 1 << split_shift; // a power of two: no integer division anywhere on the way to the first load
+	const int gstrip = static_cast<int>(blockIdx.x >> split_shift); // strip index over all segments
+	const int split	 = static_cast<int>(blockIdx.x) & (splits - 1);
+	const int sidx	 = (gstrip >= seg.strip_end[0]) + (gstrip >= seg.strip_end[1]);
+	const int strip	 = gstrip - (sidx == 0 ? 0 : seg.strip_end[sidx - 1]);
+	const int N		 = seg.rows[sidx];
+	const int slot	 = split * GEMV_WAVES + wave; // this wave's share of the strip's K range:
+	const int g0	 = slot * groups_per_slot + min(slot, groups_rem); // groups = slots * groups_per_slot + groups_rem,
+	const int g1	 = g0 + groups_per_slot + (slot < groups_rem ? 1 : 0); // the first groups_rem slots take one extra
+
+	const uint8_t* w_strip = DUMP == DUMP_X ? nullptr : seg.W[sidx] + macro_offset(strip, 0, groups);
+	const int row_l		   = strip * STRIP_ROWS + (lane & 31);
+	float acc			   = 0.0f;
+	if constexpr (!LOOP) {
+		// the host picked splits so that g1 - g0 <= TILES: straight-line code, every load of the wave in flight at once
+		acc = gemv_chunk<TILES, XF32, DUMP>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0);
+	} else {
+		// K too long for that within the host's scratch limits: walk the range in chunks of TILES groups
+		for (int gc = g0; gc < g1; gc += TILES) {
+			acc += gemv_chunk<TILES, XF32, DUMP>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0);
+			__builtin_amdgcn_wave_barrier(); // the next chunk overwrites this wave's LDS slice
+		}
+	}
+	if constexpr (DUMP != DUMP_NONE) {
 		return;
 	}
 
-	// ---- 5. one reduction per workgroup, fixed order ----
+	// ---- one reduction per workgroup, fixed order ----
 	red[wave][lane] = acc;
 	__syncthreads();
 	float total = 0.0f;
@@ -239,6 +300,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(const uint8
 		}
 	}
 	const int row = strip * STRIP_ROWS + tid;
+	float* y	  = seg.y[sidx];
 	if (splits == 1) {
 		if (tid < STRIP_ROWS && row < N) {
 			y[row] = total;
@@ -246,21 +308,21 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(const uint8
 		return;
 	}
 
-	// ---- 6. K split over several workgroups: publish partial sums, the last arriver adds them in split order ----
+	// ---- K split over several workgroups: publish partial sums, the last arriver adds them in split order ----
 	// Each XCD has its own L2, so data that crosses workgroups goes through device-scope atomic stores and loads
 	// (written through to / read from the memory side).  A device-wide fence would also order them, but it writes
 	// back and invalidates the whole L2 under the other workgroups' streaming loads; waiting for the stores to be
 	// acknowledged before the arrival count is bumped is all the ordering this hand-off needs.
 	if (tid < STRIP_ROWS) {
-		__hip_atomic_store(&partials[(static_cast<int64_t>(strip) * splits + split) * STRIP_ROWS + tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__hip_atomic_store(&partials[(static_cast<int64_t>(gstrip) * splits + split) * STRIP_ROWS + tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 	}
 	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // s_waitcnt only: the stores above have completed
 	__syncthreads();
 	if (tid == 0) {
-		const unsigned prev = __hip_atomic_fetch_add(&counters[strip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		const unsigned prev = __hip_atomic_fetch_add(&counters[gstrip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		const int last		= (prev == static_cast<unsigned>(splits - 1));
 		if (last) {
-			__hip_atomic_store(&counters[strip], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // all arrived: ready for the next launch
+			__hip_atomic_store(&counters[gstrip], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // all arrived: ready for the next launch
 		}
 		last_flag = last;
 	}
@@ -268,7 +330,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(const uint8
 	if (last_flag && tid < STRIP_ROWS && row < N) {
 		float sum = 0.0f;
 		for (int sp = 0; sp < splits; ++sp) {
-			sum += __hip_atomic_load(&partials[(static_cast<int64_t>(strip) * splits + sp) * STRIP_ROWS + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			sum += __hip_atomic_load(&partials[(static_cast<int64_t>(gstrip) * splits + sp) * STRIP_ROWS + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		}
 		y[row] = sum;
 	}
@@ -276,7 +338,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(const uint8
 
 // Scratch of the K-split path: partial sums and arrival counters, one allocation per device, made on first use
 // and kept for the life of the process.  Calls that overlap on one GPU (different streams) and both split K race on it.
-constexpr int GEMV_MAX_SPLIT_UNITS = 8192; // strips * splits when splits > 1
+constexpr int GEMV_MAX_SPLIT_UNITS	= 8192; // strips * splits when splits > 1
 constexpr int GEMV_MAX_SPLIT_STRIPS = 512;
 struct gemv_scratch {
 	float* partials	   = nullptr;
@@ -285,7 +347,7 @@ struct gemv_scratch {
 static hipError_t get_gemv_scratch(gemv_scratch* out) {
 	static std::mutex lock;
 	static gemv_scratch per_device[64];
-	int dev = 0;
+	int dev		 = 0;
 	hipError_t e = hipGetDevice(&dev);
 	if (e != hipSuccess) {
 		return e;
@@ -314,31 +376,88 @@ static hipError_t get_gemv_scratch(gemv_scratch* out) {
 	return hipSuccess;
 }
 
-// How a [N x K] tiled mat-vec is cut: `splits` workgroups per strip, each of 16 waves owning <= `tiles` groups.
+// How a tiled mat-vec launch is cut: `splits` workgroups per strip, each of 16 waves owning <= `tiles` groups.
 struct gemv_plan {
 	int strips, groups, splits, tiles;
 };
-static gemv_plan plan_gemv(int64_t N, int64_t K) {
+static gemv_plan plan_gemv(int64_t total_strips, int64_t K) {
 	gemv_plan p;
-	p.strips = static_cast<int>((N + STRIP_ROWS - 1) / STRIP_ROWS);
-	p.groups = static_cast<int>(K / GROUP_K);
-	p.splits = 1;
+	p.strips	   = static_cast<int>(total_strips);
+	p.groups	   = static_cast<int>(K / GROUP_K);
+	p.splits	   = 1;
 	auto tiles_for = [&](int s) { return (p.groups + GEMV_WAVES * s - 1) / (GEMV_WAVES * s); };
 	// split further while a wave would own more than 4 groups, or while the grid cannot cover the chip and waves still own > 1 group
-	while ((tiles_for(p.splits) > 4 || (p.strips * p.splits < 256 && GEMV_WAVES * p.splits < p.groups)) && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS && p.strips <= GEMV_MAX_SPLIT_STRIPS) {
+	while ((tiles_for(p.splits) > 4 || (p.strips * p.splits < 256 && GEMV_WAVES * p.splits < p.groups)) && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS &&
+		p.strips <= GEMV_MAX_SPLIT_STRIPS) {
 		p.splits *= 2;
 	}
 	p.tiles = tiles_for(p.splits);
 	return p;
 }
 
-template<int TILES> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const uint8_t* W, const uint8_t* xq, float* y, int32_t* sums, const gemv_scratch& sc, int N, hipStream_t s) {
+template<int TILES, bool XF32, bool LOOP> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, hipStream_t s) {
 	const dim3 grid(static_cast<unsigned>(p.strips * p.splits)), block(GEMV_WAVES * 64);
-	if (sums) {
-		gemv_tiled_kernel<TILES, true><<<grid, block, 0, s>>>(W, xq, y, sums, sc.partials, sc.counters, N, p.groups, p.splits);
+	int shift = 0;
+	while ((1 << shift) < p.splits) {
+		++shift;
+	}
+	const int slots = p.splits * GEMV_WAVES, per_slot = p.groups / slots, rem = p.groups % slots;
+	if (dump_mode == DUMP_SUMS) {
+		gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, false>, grid, block, 0, s, W, xq, y, sums, sc.partials, sc.counters, N, p.groups, p.splits);
+	if (dump_mode == DUMP_X) {
+		gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem);
+		return hipGetLastError();
+	}
+	return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP>, grid, block, 0, s, seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem);
+}
+
+static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, void* dump, int dump_mode, hipStream_t s) {
+	gemv_segments seg{};
+	int64_t strips = 0;
+	for (int i = 0; i < GEMV_MAX_SEGMENTS; ++i) {
+		if (i < count) {
+			seg.W[i]	= static_cast<const uint8_t*>(W[i]);
+			seg.y[i]	= y ? y[i] : nullptr;
+			seg.rows[i] = static_cast<int>(N[i]);
+			strips += (N[i] + STRIP_ROWS - 1) / STRIP_ROWS;
+		}
+		seg.strip_end[i] = static_cast<int>(strips);
+	}
+	if (strips == 0) {
+		return hipSuccess;
+	}
+	const gemv_plan p = plan_gemv(strips, K);
+	gemv_scratch sc;
+	if (p.splits > 1) {
+		const hipError_t e = get_gemv_scratch(&sc);
+		if (e != hipSuccess) {
+			return e;
+		}
+	}
+	if (p.tiles > 4) { // K too long to keep every load in flight within the scratch limits: chunked walk
+		return x_is_f32 ? launch_gemv_tiled_t<4, true, true>(p, seg, x, dump, dump_mode, sc, s) : launch_gemv_tiled_t<4, false, true>(p, seg, x, dump, dump_mode, sc, s);
+	}
+	const int tiles = p.tiles <= 1 ? 1 : (p.tiles <= 2 ? 2 : 4);
+	if (x_is_f32) {
+		switch (tiles) {
+			case 1:
+				return launch_gemv_tiled_t<1, true, false>(p, seg, x, dump, dump_mode, sc, s);
+			case 2:
+				return launch_gemv_tiled_t<2, true, false>(p, seg, x, dump, dump_mode, sc, s);
+			default:
+				return launch_gemv_tiled_t<4, true, false>(p, seg, x, dump, dump_mode, sc, s);
+		}
+	}
+	switch (tiles) {
+		case 1:
+			return launch_gemv_tiled_t<1, false, false>(p, seg, x, dump, dump_mode, sc, s);
+		case 2:
+			return launch_gemv_tiled_t<2, false, false>(p, seg, x, dump, dump_mode, sc, s);
+		default:
+			return launch_gemv_tiled_t<4, false, false>(p, seg, x, dump, dump_mode, sc, s);
+	}
 }
 
 // y <- 0 for an empty inner dimension (a fill kernel rather than a memset node, so the call can be graph-captured)
@@ -349,14 +468,14 @@ __global__ void zero_f32_kernel(float* __restrict__ y, int64_t n) {
 	}
 }
 
-template<int WAVES, bool TILED> static hipError_t launch_gemv_t(const uint8_t* W, const uint8_t* xq, float* y, int32_t* sums, int N, int K, hipStream_t s) {
+template<int WAVES> static hipError_t launch_gemv_blocks_t(const uint8_t* W, const uint8_t* xq, float* y, int32_t* sums, int N, int K, hipStream_t s) {
 	const int strips   = (N + STRIP_ROWS - 1) / STRIP_ROWS;
 	const size_t shmem = static_cast<size_t>(K) + static_cast<size_t>(K / QK) * 4 + WAVES * 64 * 4;
 	if (sums) {
-		gemv_kernel<WAVES, TILED, true><<<dim3(strips), dim3(WAVES * 64), shmem, s>>>(W, xq, y, sums, N, K);
+		gemv_blocks_kernel<WAVES, true><<<dim3(strips), dim3(WAVES * 64), shmem, s>>>(W, xq, y, sums, N, K);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMV, gemv_kernel<WAVES, TILED, false>, dim3(strips), dim3(WAVES * 64), shmem, s, W, xq, y, sums, N, K);
+	return launch_kernel(KIND_GEMV, gemv_blocks_kernel<WAVES, false>, dim3(strips), dim3(WAVES * 64), shmem, s, W, xq, y, sums, N, K);
 }
 
 hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* sums, int64_t N, int64_t K, bool tiled, hipStream_t s) {
@@ -370,29 +489,29 @@ hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* 
 	const uint8_t* w = static_cast<const uint8_t*>(W);
 	const uint8_t* x = static_cast<const uint8_t*>(xq_blocks);
 	if (tiled) {
-		const gemv_plan p = plan_gemv(N, K);
-		if (p.tiles <= 4) {
-			gemv_scratch sc;
-			if (p.splits > 1) {
-				const hipError_t e = get_gemv_scratch(&sc);
-				if (e != hipSuccess) {
-					return e;
-				}
-			}
-			const int n = static_cast<int>(N);
-			switch (p.tiles) {
-				case 1:
-					return launch_gemv_tiled_t<1>(p, w, x, y, sums, sc, n, s);
-				case 2:
-					return launch_gemv_tiled_t<2>(p, w, x, y, sums, sc, n, s);
-				default:
-					return launch_gemv_tiled_t<4>(p, w, x, y, sums, sc, n, s);
+		const void* wl[1] = { W };
+		float* yl[1]	  = { y };
+		return launch_gemv_tiled_any(wl, yl, &N, 1, xq_blocks, false, K, sums, sums ? DUMP_SUMS : DUMP_NONE, s);
+	}
+	return launch_gemv_blocks_t<4>(w, x, y, sums, static_cast<int>(N), static_cast<int>(K), s);
+}
+
+hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s) {
+	if (K == 0) {
+		for (int i = 0; i < count; ++i) {
+			if (N[i] > 0) {
+				zero_f32_kernel<<<dim3(static_cast<unsigned>((N[i] + 255) / 256)), dim3(256), 0, s>>>(y[i], N[i]);
 			}
 		}
-		// K too long to split within the scratch limits: the looping kernel takes it
-		return launch_gemv_t<4, true>(w, x, y, sums, static_cast<int>(N), static_cast<int>(K), s);
+		return hipGetLastError();
 	}
-	return launch_gemv_t<4, false>(w, x, y, sums, static_cast<int>(N), static_cast<int>(K), s);
+	return launch_gemv_tiled_any(W, y, N, count, x, x_is_f32, K, nullptr, DUMP_NONE, s);
+}
+
+hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s) {
+	const void* wl[1] = { nullptr }; // the dump variant never touches the weights
+	const int64_t n	  = STRIP_ROWS;
+	return launch_gemv_tiled_any(wl, nullptr, &n, 1, x, true, K, xq_blocks_out, DUMP_X, s);
 }
 
 } // namespace nh

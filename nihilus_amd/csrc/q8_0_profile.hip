@@ -140,17 +140,40 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 			return NH_ERR_NULL_POINTER;
 		}
 	}
-	const float* quantized_x = nullptr; // activation currently held in the workspace
+	const float* quantized_x = nullptr; // activation currently held in the workspace (M > 1 only)
 	int64_t quantized_m = -1, quantized_k = -1;
-	for (int64_t i = 0; i < count; ++i) {
+	for (int64_t i = 0; i < count;) {
 		const nh_q8_0_mul_mat_op& op = host_ops[i];
 		if (op.M == 0 || op.N == 0) {
+			++i;
 			continue;
 		}
-		int rc				= NH_OK;
+		if (op.M == 1) {
+			// decode: the quantize lives inside the mat-vec kernel; neighbours that share x and K become one launch
+			const void* w[nh::GEMV_MAX_SEGMENTS];
+			float* y[nh::GEMV_MAX_SEGMENTS];
+			int64_t n[nh::GEMV_MAX_SEGMENTS];
+			int64_t g = 0;
+			while (i + g < count && g < nh::GEMV_MAX_SEGMENTS) {
+				const nh_q8_0_mul_mat_op& o = host_ops[i + g];
+				if (o.M != 1 || o.N == 0 || o.x != op.x || o.K != op.K || (g > 0 && !o.reuse_quantized_x)) {
+					break;
+				}
+				w[g] = o.W_tiled;
+				y[g] = o.y;
+				n[g] = o.N;
+				++g;
+			}
+			const int rc = nh_q8_0_gemv_tiled_multi_f32(w, y, n, g, op.x, op.K, stream);
+			if (rc != NH_OK) {
+				return rc;
+			}
+			i += g;
+			continue;
+		}
 		const bool reuse = op.reuse_quantized_x && quantized_x == op.x && quantized_m == op.M && quantized_k == op.K;
 		if (!reuse) {
-			rc = (op.M == 1) ? nh_q8_0_quantize(op.x, workspace, 1, op.K, stream) : nh_q8_0_quantize_tiled(op.x, workspace, op.M, op.K, stream);
+			const int rc = nh_q8_0_quantize_tiled(op.x, workspace, op.M, op.K, stream);
 			if (rc != NH_OK) {
 				return rc;
 			}
@@ -158,10 +181,11 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 			quantized_m = op.M;
 			quantized_k = op.K;
 		}
-		rc = (op.M == 1) ? nh_q8_0_gemv_tiled(op.W_tiled, workspace, op.y, op.N, op.K, stream) : nh_q8_0_gemm_tiled(op.W_tiled, workspace, op.y, op.M, op.N, op.K, stream);
+		const int rc = nh_q8_0_gemm_tiled(op.W_tiled, workspace, op.y, op.M, op.N, op.K, stream);
 		if (rc != NH_OK) {
 			return rc;
 		}
+		++i;
 	}
 	return NH_OK;
 }

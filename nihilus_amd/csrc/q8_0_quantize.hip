@@ -26,24 +26,8 @@ template<bool TILED> __global__ __launch_bounds__(256) void quantize_kernel(cons
 	if (in_range && m < M) {
 		v = *reinterpret_cast<const float4*>(x + m * K + b * QK + 4 * j);
 	}
-	float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-	amax	   = fmaxf(amax, __shfl_xor(amax, 1));
-	amax	   = fmaxf(amax, __shfl_xor(amax, 2));
-	amax	   = fmaxf(amax, __shfl_xor(amax, 4));
-
-	const float d	  = __fdiv_rn(amax, 127.0f);
-	const float id	  = (amax != 0.0f) ? __fdiv_rn(127.0f, amax) : 0.0f;
-	const uint16_t dh = float_to_half_bits(d);
-
-	auto q8 = [id](float f) -> uint32_t {
-		const float r = rintf(__fmul_rn(f, id)); // v_rndne_f32: ties to even
-		// x86 cvtps_epi32 yields 0x80000000 for NaN and out-of-range values, which the reference's saturating packs
-		// turn into -128.  Reachable only when 127/amax overflows to inf (amax below ~3.7e-37): inf, and 0*inf = NaN.
-		int q = (fabsf(r) < 2147483648.0f) ? static_cast<int>(r) : INT32_MIN;
-		q	  = max(-128, min(127, q));
-		return static_cast<uint32_t>(q) & 0xFFu;
-	};
-	const uint32_t packed = q8(v.x) | (q8(v.y) << 8) | (q8(v.z) << 16) | (q8(v.w) << 24);
+	uint16_t dh;
+	const uint32_t packed = quantize_block_lane(v, &dh);
 
 	if (!in_range) {
 		return;

@@ -80,6 +80,37 @@ def gemv(w: torch.Tensor, xq_blocks: torch.Tensor, n: int, k: int, tiled: bool) 
     return y
 
 
+def gemv_f32(w_tiled: list[torch.Tensor] | torch.Tensor, x: torch.Tensor, n: list[int] | int, k: int) -> list[torch.Tensor] | torch.Tensor:
+    """Fused quantize + mat-vec on tiled weights; a list of up to 3 weights sharing x and k runs as one launch."""
+    import ctypes as C
+
+    single = not isinstance(w_tiled, (list, tuple))
+    ws = [w_tiled] if single else list(w_tiled)
+    ns = [n] if single else list(n)
+    x = _dev(x, torch.float32, "x")
+    if x.numel() != k or len(ws) != len(ns):
+        raise ValueError("x must hold k floats and every weight needs its row count")
+    for w, nn in zip(ws, ns):
+        if _dev(w, torch.uint8, "w_tiled").numel() != tiled_bytes(nn, k):
+            raise ValueError("weight size does not match n x k")
+    ys = [torch.empty(nn, dtype=torch.float32, device=x.device) for nn in ns]
+    cnt = len(ws)
+    wp = (C.c_void_p * cnt)(*[w.data_ptr() for w in ws])
+    yp = (C.c_void_p * cnt)(*[y.data_ptr() for y in ys])
+    np_ = (C.c_int64 * cnt)(*ns)
+    _lib.check("nh_q8_0_gemv_tiled_multi_f32", _lib.lib().nh_q8_0_gemv_tiled_multi_f32(wp, yp, np_, cnt, x.data_ptr(), k, _stream()))
+    return ys[0] if single else ys
+
+
+def debug_fused_quantize(x: torch.Tensor) -> torch.Tensor:
+    """The activation row exactly as the fused mat-vec stages it, as packed blocks."""
+    x = _dev(x, torch.float32, "x")
+    k = x.numel()
+    out = torch.zeros(blocks_bytes(1, k), dtype=torch.uint8, device=x.device)
+    _lib.check("nh_q8_0_debug_fused_quantize", _lib.lib().nh_q8_0_debug_fused_quantize(x.data_ptr(), out.data_ptr(), k, _stream()))
+    return out
+
+
 def gemm(w: torch.Tensor, aq: torch.Tensor, m: int, n: int, k: int, tiled: bool) -> torch.Tensor:
     w, aq = _dev(w, torch.uint8, "w"), _dev(aq, torch.uint8, "aq")
     size = tiled_bytes if tiled else blocks_bytes

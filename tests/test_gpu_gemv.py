@@ -83,7 +83,7 @@ def test_gemv_errors(q8):
     assert lib.nh_q8_0_gemv_tiled(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 96, None) == -3
     assert lib.nh_q8_0_gemv(None, xq.data_ptr(), y.data_ptr(), 32, 128, None) == -1
     assert lib.nh_q8_0_gemv(w.data_ptr() + 2, xq.data_ptr(), y.data_ptr(), 32, 128, None) == -2
-    assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 1 << 20, None) == -5
+    assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 1 << 20, None) == -5  # blocks-layout mat-vec: K bounded by LDS
     torch.cuda.synchronize()
     assert bool((y == 7.0).all())  # rejected calls wrote nothing
     assert lib.nh_q8_0_gemv(w.data_ptr(), xq.data_ptr(), y.data_ptr(), 32, 0, None) == 0  # empty dot product
@@ -101,3 +101,47 @@ def test_gemv_split_k_is_deterministic_and_reusable(q8, oracle):
     for _ in range(20):
         assert np.array_equal(to_host(q8.gemv(wt, xqd, n, k, tiled=True)), first)
     assert rel_l2(first, oracle.gemv(w, xq, n, k)) <= REL_L2_TOL
+
+
+@pytest.mark.parametrize("k", [128, 4096, 14336, 28672, 512 * 128])
+def test_fused_quantize_stage_is_bit_exact(q8, oracle, k):
+    # the quantize inside the mat-vec kernel must stage exactly the bytes the stand-alone quantizer writes
+    rng = np.random.default_rng(k)
+    for x in (oracle.fill_activations(k, k), (rng.standard_normal(k) * 2.0 ** rng.integers(-30, 30, size=k)).astype(np.float32)):
+        got = to_host(q8.debug_fused_quantize(to_dev(x)))
+        assert np.array_equal(got, oracle.quantize_rows(x)[0])
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (14336, 4096), (4096, 14336), (33, 128), (8192, 28672)])
+def test_gemv_fused_f32_equals_two_step(q8, oracle, n, k):
+    w, x, xq = _inputs(oracle, n, k, seed=n + 3 * k)
+    wt = q8.tile(to_dev(w), n, k)
+    fused = to_host(q8.gemv_f32(wt, to_dev(x), n, k))
+    two_step = to_host(q8.gemv(wt, to_dev(xq), n, k, tiled=True))
+    assert np.array_equal(fused, two_step)  # same staged bytes, same kernel, same order
+    assert rel_l2(fused, oracle.gemv(w, xq, n, k)) <= REL_L2_TOL
+
+
+def test_gemv_multi_segment(q8, oracle):
+    # q/k/v-shaped and gate/up-shaped groups as one launch each; results equal the single launches bit for bit
+    for ns, k in [([4096, 1024, 1024], 4096), ([14336, 14336], 4096), ([40, 33, 1], 256), ([96], 128)]:
+        x = oracle.fill_activations(9, k)
+        ws = [oracle.fill_weights(50 + i, n, k) for i, n in enumerate(ns)]
+        wts = [q8.tile(to_dev(w), n, k) for w, n in zip(ws, ns)]
+        xd = to_dev(x)
+        ys = q8.gemv_f32(wts, xd, ns, k)
+        xq = oracle.quantize_rows(x)[0]
+        for w, wt, n, y in zip(ws, wts, ns, ys):
+            assert rel_l2(to_host(y), oracle.gemv(w, xq, n, k)) <= REL_L2_TOL
+            if sum((m + 31) // 32 for m in ns) >= 256 or len(ns) == 1:  # same K split as the single launch
+                assert np.array_equal(to_host(y), to_host(q8.gemv_f32(wt, xd, n, k)))
+
+
+def test_gemv_long_k_many_rows_chunked_walk(q8, oracle):
+    # many strips AND a K too long for one pass per wave: the kernel walks its K range in chunks
+    n, k = 16416, 16384  # 513 strips (> split limit), 128 groups -> 8 groups per wave
+    w, x, xq = _inputs(oracle, n, k, seed=4)
+    wt = q8.tile(to_dev(w), n, k)
+    want = oracle.gemm(w, xq[None, :], 1, n, k, threads=8)[0]
+    assert rel_l2(to_host(q8.gemv(wt, to_dev(xq), n, k, tiled=True)), want) <= REL_L2_TOL
+    assert rel_l2(to_host(q8.gemv_f32(wt, to_dev(x), n, k)), want) <= REL_L2_TOL
