@@ -25,6 +25,9 @@ HIPCC_FLAGS = [
     "-Wall",
     "-Wextra",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results stay in ordinary VGPRs: the mat-mat converts every int32 block sum on the VALU right away, and a
+    # result parked in an accumulation register would cost one extra copy instruction per value (doubling the VALU work)
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 
