@@ -115,5 +115,8 @@ hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const 
 // Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s);
 hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s);
+// Tiled operands, M <= GEMM_SKINNY_MAX_M: the HBM-streaming MFMA kernel for batched decode (q8_0_gemm_skinny.hip).
+constexpr int64_t GEMM_SKINNY_MAX_M = 64;
+hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s);
 
 } // namespace nh

@@ -424,6 +424,9 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 	const uint8_t* a = static_cast<const uint8_t*>(Aq);
 	const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
 	if (tiled) {
+		if (M <= GEMM_SKINNY_MAX_M) {
+			return launch_gemm_skinny(W, Aq, C, sums, M, N, K, s); // few rows: weights are read once, the kernel is HBM-bound
+		}
 		return launch_gemm_tiled(w, a, C, sums, m, n, k, s);
 	} else {
 		if (sums) {

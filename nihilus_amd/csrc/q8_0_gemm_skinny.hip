@@ -1,0 +1,303 @@
+// Batched-decode mat-mat for a handful of activation rows (M <= 64): C[m][n] = dot(W row n, Aq row m), gfx950.
+//
+// With so few rows the weights are read once and nothing is reused enough to leave the HBM roofline, so this is the
+// streaming mat-vec again -- one workgroup per (32-row weight strip, K split), waves splitting the strip's K range,
+// all of a chunk's loads issued before anything is waited for, one fixed-order reduction at the end -- with the
+// v_dot4 inner product replaced by the int8 MFMA: the weight tile a wave fetches (one coalesced 16-byte-per-lane load
+// in the tiled layout) is the B operand as it stands, the matching activation tile (served by L2: the activations
+// are M*K bytes) is the A operand, and one v_mfma_i32_32x32x32_i8 yields the exact block sums of 32 rows x 32
+// columns.  Scale products come from a v_mfma_f32_32x32x8_f16 on the blocks' fp16 scales (exact, same register layout),
+// then one convert + one multiply-add per value.  Same arithmetic as the prefill kernel (reference
+// vec_dot_q8_0_q8_0, cpu/avx_2.hpp:4534-4747; output [M][N], n fastest, cpu/avx_2.hpp:4934).
+#include "q8_0_device.h"
+
+#include <mutex>
+
+namespace nh {
+
+constexpr int SK_WAVES = 8;
+constexpr int SK_TILES = 1; // 128-quant groups per chunk: loads of one chunk are all in flight together; one keeps the
+                            // register count low enough for two workgroups per CU, so one computes while the other waits on loads
+
+typedef _Float16 sk_v4h __attribute__((ext_vector_type(4)));
+typedef float sk_v16f __attribute__((ext_vector_type(16)));
+
+// fp16 scale of block t (0..3) from a row's four packed scales, as the f16 MFMA's k = 0 slot: {d_t, 0, 0, 0}
+__device__ __forceinline__ v2u scale_slot(v2u four, int t) {
+	const uint32_t dword = (t < 2) ? four.x : four.y;
+	return v2u{ (t & 1) ? (dword >> 16) : (dword & 0xFFFFu), 0u };
+}
+
+template<int MS, bool DUMP>
+__global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums,
+	float* __restrict__ partials, unsigned* __restrict__ counters, int M, int N, int groups, int split_shift, int groups_per_slot, int groups_rem) {
+	__shared__ float red[SK_WAVES / 2][MS][16][64];
+	__shared__ int last_flag;
+
+	const int tid	 = threadIdx.x;
+	const int lane	 = tid & 63;
+	const int wave	 = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int splits = 1 << split_shift;
+	const int strip	 = static_cast<int>(blockIdx.x >> split_shift);
+	const int split	 = static_cast<int>(blockIdx.x) & (splits - 1);
+	const int slot	 = split * SK_WAVES + wave;
+	const int g0	 = slot * groups_per_slot + min(slot, groups_rem);
+	const int g1	 = g0 + groups_per_slot + (slot < groups_rem ? 1 : 0);
+	const int r		 = lane & 31;
+	const int half	 = lane >> 5;
+
+	sk_v16f acc[MS];
+#pragma unroll
+	for (int i = 0; i < MS; ++i) {
+		acc[i] = sk_v16f{ 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+	}
+
+	const uint8_t* w_strip = W + macro_offset(strip, 0, groups);
+	for (int gc = g0; gc < g1; gc += SK_TILES) {
+		const int cnt = min(SK_TILES, g1 - gc);
+		// ---- every byte of the chunk in flight: weight tiles (HBM, non-temporal) and activation tiles (L2) ----
+		v4i wq[SK_TILES][GROUP_BLOCKS], aq[SK_TILES][MS][GROUP_BLOCKS];
+		v2u wd[SK_TILES], ad[SK_TILES][MS];
+#pragma unroll
+		for (int t = 0; t < SK_TILES; ++t) {
+			if (t < cnt) {
+				const uint8_t* macro = w_strip + static_cast<int64_t>(gc + t) * MACRO_BYTES;
+#pragma unroll
+				for (int j = 0; j < GROUP_BLOCKS; ++j) {
+					wq[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+				}
+				wd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+#pragma unroll
+				for (int i = 0; i < MS; ++i) {
+					const uint8_t* am = A + macro_offset(i, gc + t, groups);
+#pragma unroll
+					for (int j = 0; j < GROUP_BLOCKS; ++j) {
+						aq[t][i][j] = *reinterpret_cast<const v4i*>(am + j * TILE_BYTES + 16 * lane);
+					}
+					ad[t][i] = *reinterpret_cast<const v2u*>(am + MACRO_D_OFFSET + 8 * r);
+				}
+			}
+		}
+		// ---- MFMA per block, fold per block ----
+#pragma unroll
+		for (int t = 0; t < SK_TILES; ++t) {
+			if (t < cnt) {
+				// lanes 32..63 feed the k = 4..7 slots of the scale MFMA: zero
+				const v2u wdz = half ? v2u{ 0u, 0u } : wd[t];
+#pragma unroll
+				for (int j = 0; j < GROUP_BLOCKS; ++j) {
+					const v2u ws = scale_slot(wdz, j);
+#pragma unroll
+					for (int i = 0; i < MS; ++i) {
+						const sk_v16f zf = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+						const v16i zi	 = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+						const v16i s	 = __builtin_amdgcn_mfma_i32_32x32x32_i8(aq[t][i][j], wq[t][j], zi, 0, 0, 0);
+						if constexpr (DUMP) {
+							const int n = strip * STRIP_ROWS + r;
+#pragma unroll
+							for (int e = 0; e < 16; ++e) {
+								const int m = i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+								if (m < M && n < N) {
+									sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + ((gc + t) * GROUP_BLOCKS + j)] = s[e];
+								}
+							}
+						} else {
+							const v2u as	= scale_slot(half ? v2u{ 0u, 0u } : ad[t][i], j);
+							const sk_v16f p = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(sk_v4h, as), __builtin_bit_cast(sk_v4h, ws), zf, 0, 0, 0);
+#pragma unroll
+							for (int e = 0; e < 16; ++e) {
+								acc[i][e] = fmaf(static_cast<float>(s[e]), p[e], acc[i][e]);
+							}
+						}
+					}
+				}
+			}
+		}
+	}
+	if constexpr (DUMP) {
+		return;
+	}
+
+	// ---- fixed-order tree reduction over the workgroup's waves ----
+#pragma unroll
+	for (int s = SK_WAVES / 2; s >= 1; s >>= 1) {
+		if (wave >= s && wave < 2 * s) {
+#pragma unroll
+			for (int i = 0; i < MS; ++i) {
+#pragma unroll
+				for (int e = 0; e < 16; ++e) {
+					red[wave - s][i][e][lane] = acc[i][e];
+				}
+			}
+		}
+		__syncthreads();
+		if (wave < s) {
+#pragma unroll
+			for (int i = 0; i < MS; ++i) {
+#pragma unroll
+				for (int e = 0; e < 16; ++e) {
+					acc[i][e] += red[wave][i][e][lane];
+				}
+			}
+		}
+		__syncthreads();
+	}
+
+	const int n = strip * STRIP_ROWS + r;
+	if (splits == 1) {
+		if (wave == 0 && n < N) {
+#pragma unroll
+			for (int i = 0; i < MS; ++i) {
+#pragma unroll
+				for (int e = 0; e < 16; ++e) {
+					const int m = i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+					if (m < M) {
+						C[static_cast<int64_t>(m) * N + n] = acc[i][e];
+					}
+				}
+			}
+		}
+		return;
+	}
+
+	// ---- K split over several workgroups: partial tiles through device-scope atomics, last arriver adds in split order ----
+	float* mine = partials + (static_cast<int64_t>(strip) * splits + split) * (MS * 16 * 64);
+	if (wave == 0) {
+#pragma unroll
+		for (int i = 0; i < MS; ++i) {
+#pragma unroll
+			for (int e = 0; e < 16; ++e) {
+				__hip_atomic_store(&mine[(i * 16 + e) * 64 + lane], acc[i][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
+		}
+	}
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // the stores have completed (written through) before the arrival is counted
+	__syncthreads();
+	if (tid == 0) {
+		const unsigned prev = __hip_atomic_fetch_add(&counters[strip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		const int last		= (prev == static_cast<unsigned>(splits - 1));
+		if (last) {
+			__hip_atomic_store(&counters[strip], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		}
+		last_flag = last;
+	}
+	__syncthreads();
+	if (last_flag && wave == 0 && n < N) {
+		// two splits' worth of partial tiles requested at a time (32 loads per lane in flight), added in split order
+		sk_v16f sum[MS];
+#pragma unroll
+		for (int i = 0; i < MS; ++i) {
+			sum[i] = sk_v16f{ 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+		}
+		const float* base = partials + static_cast<int64_t>(strip) * splits * (MS * 16 * 64) + lane;
+#pragma unroll
+		for (int i = 0; i < MS; ++i) {
+			for (int sp0 = 0; sp0 < splits; sp0 += 2) {
+				float v[2][16];
+#pragma unroll
+				for (int u = 0; u < 2; ++u) {
+#pragma unroll
+					for (int e = 0; e < 16; ++e) {
+						v[u][e] = (sp0 + u < splits) ? __hip_atomic_load(&base[(static_cast<int64_t>(sp0 + u) * (MS * 16) + (i * 16 + e)) * 64], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+					}
+				}
+#pragma unroll
+				for (int u = 0; u < 2; ++u) {
+					if (sp0 + u < splits) {
+#pragma unroll
+						for (int e = 0; e < 16; ++e) {
+							sum[i][e] += v[u][e];
+						}
+					}
+				}
+			}
+#pragma unroll
+			for (int e = 0; e < 16; ++e) {
+				const int m = i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+				if (m < M) {
+					C[static_cast<int64_t>(m) * N + n] = sum[i][e];
+				}
+			}
+		}
+	}
+}
+
+// Scratch of the K-split path (partial 32x32 tiles and arrival counters): one allocation per device on first use.
+constexpr int SK_MAX_SPLIT_UNITS  = 2048; // strips * splits when splits > 1
+constexpr int SK_MAX_SPLIT_STRIPS = 512;
+struct skinny_scratch {
+	float* partials	   = nullptr;
+	unsigned* counters = nullptr;
+};
+static hipError_t get_skinny_scratch(skinny_scratch* out) {
+	static std::mutex lock;
+	static skinny_scratch per_device[64];
+	int dev		 = 0;
+	hipError_t e = hipGetDevice(&dev);
+	if (e != hipSuccess) {
+		return e;
+	}
+	if (dev < 0 || dev >= 64) {
+		return hipErrorInvalidDevice;
+	}
+	std::lock_guard<std::mutex> g(lock);
+	skinny_scratch& sc = per_device[dev];
+	if (!sc.partials) {
+		void* p			   = nullptr;
+		const size_t tiles = static_cast<size_t>(SK_MAX_SPLIT_UNITS) * 2 * 16 * 64 * 4; // two 32-row activation strips at most
+		const size_t bytes = tiles + SK_MAX_SPLIT_STRIPS * 4;
+		e				   = hipMalloc(&p, bytes);
+		if (e != hipSuccess) {
+			return e;
+		}
+		e = hipMemset(p, 0, bytes);
+		if (e != hipSuccess) {
+			(void)hipFree(p);
+			return e;
+		}
+		sc.partials = static_cast<float*>(p);
+		sc.counters = reinterpret_cast<unsigned*>(static_cast<uint8_t*>(p) + tiles);
+	}
+	*out = sc;
+	return hipSuccess;
+}
+
+template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int groups, hipStream_t s) {
+	const int strips = (n + STRIP_ROWS - 1) / STRIP_ROWS;
+	int splits		 = 1;
+	// The hand-off between workgroups costs a few microseconds, so K is split over workgroups only when a wave would
+	// otherwise walk more than four groups one after the other (few rows, long K: the down projections).
+	while (groups > 4 * SK_WAVES * splits && strips * splits * 2 <= SK_MAX_SPLIT_UNITS && strips <= SK_MAX_SPLIT_STRIPS) {
+		splits *= 2;
+	}
+	skinny_scratch sc;
+	if (splits > 1) {
+		const hipError_t e = get_skinny_scratch(&sc);
+		if (e != hipSuccess) {
+			return e;
+		}
+	}
+	int shift = 0;
+	while ((1 << shift) < splits) {
+		++shift;
+	}
+	const int slots = splits * SK_WAVES, per_slot = groups / slots, rem = groups % slots;
+	const dim3 grid(static_cast<unsigned>(strips * splits)), block(SK_WAVES * 64);
+	if (sums) {
+		gemm_skinny_kernel<MS, true><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+		return hipGetLastError();
+	}
+	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+}
+
+hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+	const uint8_t* w = static_cast<const uint8_t*>(W);
+	const uint8_t* a = static_cast<const uint8_t*>(Aq);
+	const int groups = static_cast<int>(K / GROUP_K);
+	if (M <= 32) {
+		return launch_skinny_t<1>(w, a, C, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
+	}
+	return launch_skinny_t<2>(w, a, C, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
+}
+
+} // namespace nh

@@ -328,9 +328,22 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	}
 	__syncthreads();
 	if (last_flag && tid < STRIP_ROWS && row < N) {
-		float sum = 0.0f;
-		for (int sp = 0; sp < splits; ++sp) {
-			sum += __hip_atomic_load(&partials[(static_cast<int64_t>(gstrip) * splits + sp) * STRIP_ROWS + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		// all partial sums requested before the first is waited for (they come from the memory side, ~1 us each if
+		// taken one at a time), then added in split order
+		const float* mine = partials + static_cast<int64_t>(gstrip) * splits * STRIP_ROWS + tid;
+		float sum		  = 0.0f;
+		for (int sp0 = 0; sp0 < splits; sp0 += 8) {
+			float v[8];
+#pragma unroll
+			for (int u = 0; u < 8; ++u) {
+				v[u] = (sp0 + u < splits) ? __hip_atomic_load(&mine[(sp0 + u) * STRIP_ROWS], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+			}
+#pragma unroll
+			for (int u = 0; u < 8; ++u) {
+				if (sp0 + u < splits) {
+					sum += v[u];
+				}
+			}
 		}
 		y[row] = sum;
 	}

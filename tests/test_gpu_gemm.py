@@ -22,7 +22,7 @@ def test_gemm_tiled_and_blocks(q8, oracle, m, n, k):
     c_tiled = to_host(q8.gemm(q8.tile(wd, n, k), q8.tile(aqd, m, k), m, n, k, tiled=True))
     assert rel_l2(c_blocks, want) <= REL_L2_TOL
     assert rel_l2(c_tiled, want) <= REL_L2_TOL
-    assert np.array_equal(c_blocks, c_tiled)
+    assert rel_l2(c_blocks, c_tiled) < 2e-6  # different kernels, different fp32 order, same exact block sums
     # every row separately, so one bad row cannot hide in the norm of the rest
     for i in range(0, m, max(1, m // 7)):
         assert rel_l2(c_tiled[i], want[i]) <= REL_L2_TOL
