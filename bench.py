@@ -60,6 +60,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
     ap.add_argument("--calibration-copies", type=int, default=0, help="run this many plain 64 MiB device copies first (a known-size kernel to scale hardware byte counters by)")
+    ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode-step leg (8 GB of weights)")
+    ap.add_argument("--decode-tokens", type=int, default=200, help="timed tokens of the decode-step leg")
     ap.add_argument("--roofline-steps", type=int, default=0, help="steps of the per-kernel timing pass (default: min(steps, 1000))")
     args = ap.parse_args()
 
@@ -107,7 +109,7 @@ def main() -> int:
     y_up = torch.empty(GATE_N, dtype=torch.float32, device=dev)
     y_down = torch.empty(HIDDEN, dtype=torch.float32, device=dev)
     ws_bytes = max(lib.nh_q8_0_mul_mat_workspace_bytes(1, HIDDEN), lib.nh_q8_0_mul_mat_workspace_bytes(1, FFN))
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
 
     OpArr = _lib.MulMatOp * 3
     op_lists = []
@@ -192,11 +194,92 @@ def main() -> int:
         },
     }
 
+    del layers, op_lists
+    torch.cuda.empty_cache()
+    if not args.no_decode:
+        result["decode"] = decode_step(args.decode_tokens)
+
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
 
     print(json.dumps(result))
     return 0
+
+
+def decode_step(tokens: int) -> dict:
+    """The second half of the metric: one decode step of a LLaMA-3-8B-shaped model with every mat-mul in Q8_0
+    (32 layers x {q, k, v, o, gate, up, down} + lm_head, random weights from the generator, fp32 N(0,1) inputs
+    per projection; mat-muls only, no attention/norm math).  One token = one native batch call of 225 projections,
+    which the runner issues as 129 launches (q/k/v and gate/up fused).  All 8 GB of weights are distinct, so every
+    token streams them from HBM."""
+    import torch
+
+    from nihilus_amd import _lib, q8_0
+
+    lib = _lib.lib()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    H, KV, F, V, LAYERS = 4096, 1024, 14336, 128256, 32
+    shapes = [("q", H, H), ("k", KV, H), ("v", KV, H), ("o", H, H), ("gate", F, H), ("up", F, H), ("down", H, F)]
+    first = 0
+
+    def make(n, k):
+        nonlocal first
+        b = q8_0.fill_weight_blocks(4, n, k, first_block=first)
+        first += n * (k // 32)
+        t = q8_0.tile(b, n, k)
+        del b
+        return t
+
+    x_attn = q8_0.fill_activations(10, H)
+    x_o = q8_0.fill_activations(11, H)
+    x_ffn = q8_0.fill_activations(12, H)
+    x_down = q8_0.fill_activations(13, F)
+    x_head = q8_0.fill_activations(14, H)
+    xin = {"q": x_attn, "k": x_attn, "v": x_attn, "o": x_o, "gate": x_ffn, "up": x_ffn, "down": x_down}
+    outs = {name: torch.empty(n, dtype=torch.float32, device=dev) for name, n, _ in shapes}
+    logits = torch.empty(V, dtype=torch.float32, device=dev)
+    weights = []
+    ops = (_lib.MulMatOp * (LAYERS * 7 + 1))()
+    i = 0
+    wbytes = 0
+    for _ in range(LAYERS):
+        for name, n, k in shapes:
+            w = make(n, k)
+            weights.append(w)
+            wbytes += n * (k // 32) * 34
+            ops[i] = _lib.MulMatOp(w.data_ptr(), xin[name].data_ptr(), outs[name].data_ptr(), 1, n, k, 1 if name in ("k", "v", "up") else 0, 0)
+            i += 1
+    w_head = make(V, H)
+    wbytes += V * (H // 32) * 34
+    ops[i] = _lib.MulMatOp(w_head.data_ptr(), x_head.data_ptr(), logits.data_ptr(), 1, V, H, 0, 0)
+    n_ops = i + 1
+    ws = torch.empty(256, dtype=torch.uint8, device=dev)
+
+    def token():
+        rc = lib.nh_q8_0_mul_mat_batch(ops, n_ops, ws.data_ptr(), ws.numel(), stream)
+        if rc != 0:
+            _lib.check("nh_q8_0_mul_mat_batch", rc)
+
+    for _ in range(10):
+        token()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(tokens):
+        token()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / tokens
+    return {
+        "tok_s": round(1.0 / sec, 1),
+        "ms_per_token": round(sec * 1e3, 4),
+        "weight_bytes_per_token": wbytes,
+        "weight_GBs": round(wbytes / sec / 1e9, 1),
+        "pct_of_hbm_peak": round(100.0 * wbytes / sec / 1e9 / HBM_PEAK_GBS, 2),
+        "projections_per_token": n_ops,
+        "launches_per_token": LAYERS * 4 + 1,
+        "tokens_timed": tokens,
+        "outputs_finite": bool(torch.isfinite(logits).all()),
+    }
 
 
 def cpu_baseline(budget_s: float) -> dict:

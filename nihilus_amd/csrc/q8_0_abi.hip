@@ -339,8 +339,8 @@ int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K) {
 	if (M < 0 || K < 0 || K % nh::GROUP_K != 0) {
 		return NH_ERR_SHAPE;
 	}
-	if (M == 1) {
-		return (nh_q8_0_blocks_bytes(1, K) + 255) / 256 * 256;
+	if (M <= 1) {
+		return 0; // one row: the quantize happens inside the mat-vec kernel, nothing is staged in memory
 	}
 	return (nh_q8_0_tiled_bytes(M, K) + 255) / 256 * 256;
 }
@@ -353,7 +353,7 @@ int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, in
 	const int64_t need = nh_q8_0_mul_mat_workspace_bytes(M, K);
 	NH_REQUIRE(workspace_bytes >= need, NH_ERR_ARGUMENT);
 	if (K > 0) {
-		NH_REQUIRE(workspace && x, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(x && (workspace || need == 0), NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(workspace) && aligned16(x), NH_ERR_ALIGNMENT);
 	}
 	if (M == 1) {

@@ -399,9 +399,15 @@ static gemv_plan plan_gemv(int64_t total_strips, int64_t K) {
 	p.groups	   = static_cast<int>(K / GROUP_K);
 	p.splits	   = 1;
 	auto tiles_for = [&](int s) { return (p.groups + GEMV_WAVES * s - 1) / (GEMV_WAVES * s); };
-	// split further while a wave would own more than 4 groups, or while the grid cannot cover the chip and waves still own > 1 group
-	while ((tiles_for(p.splits) > 4 || (p.strips * p.splits < 256 && GEMV_WAVES * p.splits < p.groups)) && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS &&
-		p.strips <= GEMV_MAX_SPLIT_STRIPS) {
+	// K goes over several workgroups only when it has to: the hand-off between workgroups costs 1-2 us, more than an
+	// idle half of the chip costs a matrix of a few MB.  So: split until a wave owns at most 4 groups (every load of the
+	// wave in flight at once), and, once splitting anyway, one step further to 2 groups per wave (measured best on the
+	// long-K down projections).
+	const bool room = p.strips <= GEMV_MAX_SPLIT_STRIPS;
+	while (tiles_for(p.splits) > 4 && room && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
+		p.splits *= 2;
+	}
+	if (p.splits > 1 && tiles_for(p.splits) > 2 && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
 		p.splits *= 2;
 	}
 	p.tiles = tiles_for(p.splits);
