@@ -60,6 +60,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
     ap.add_argument("--calibration-copies", type=int, default=0, help="run this many plain 64 MiB device copies first (a known-size kernel to scale hardware byte counters by)")
+    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize"], default="ffn_decode",
+                    help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
+                    "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode-step leg (8 GB of weights)")
     ap.add_argument("--decode-tokens", type=int, default=200, help="timed tokens of the decode-step leg")
     ap.add_argument("--roofline-steps", type=int, default=0, help="steps of the per-kernel timing pass (default: min(steps, 1000))")
@@ -80,6 +83,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     stream = torch.cuda.current_stream().cuda_stream
+    if args.workload != "ffn_decode":
+        print(json.dumps(side_workload(args.workload, args.steps, args.warmup)))
+        return 0
 
     if args.calibration_copies > 0:
         # a plain copy of known size: 64 MiB read, 64 MiB written per kernel; counters read for it give the scale
@@ -204,6 +210,77 @@ def main() -> int:
 
     print(json.dumps(result))
     return 0
+
+
+INT8_MFMA_PEAK_TOPS = 5033.0  # MI355X published dense int8 matrix rate
+
+
+def side_workload(kind: str, steps: int, warmup: int) -> dict:
+    """One JSON line for the prefill mat-mat (BASELINE config 3: M=512, W [4096x4096] and [14336x4096]) or for the
+    stand-alone activation quantize (M=512, K=4096), each against the roofline that bounds it."""
+    import torch
+
+    from nihilus_amd import _lib, q8_0
+
+    lib = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    M, K = 512, 4096
+    x = q8_0.fill_activations(0, M * K).reshape(M, K)
+    steps = min(steps, 200)
+    warmup = min(warmup, 20)
+
+    def timed(kind_id: int, fn, launches_per_step: int):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / steps
+        _lib.check("nh_profile_begin", lib.nh_profile_begin(kind_id, launches_per_step * steps))
+        for _ in range(steps):
+            fn()
+        tot, cnt, mn, mx = C.c_double(), C.c_int64(), C.c_double(), C.c_double()
+        _lib.check("nh_profile_end", lib.nh_profile_end(C.byref(tot), C.byref(cnt), C.byref(mn), C.byref(mx)))
+        return wall, tot.value / cnt.value * 1e-3, cnt.value
+
+    if kind == "quantize":
+        out = torch.empty(q8_0.tiled_bytes(M, K), dtype=torch.uint8, device=x.device)
+        nbytes = 4 * M * K + M * (K // 32) * 34
+
+        def fn():
+            _lib.check("nh_q8_0_quantize_tiled", lib.nh_q8_0_quantize_tiled(x.data_ptr(), out.data_ptr(), M, K, stream))
+
+        wall, ksec, n = timed(0, fn, 1)
+        ach = nbytes / ksec / 1e9
+        return {
+            "metric": "Q8_0 activation quantize GB/s", "value": round(nbytes / wall / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "dtype": "fp32 -> int8 + fp16 scale", "data": "synthetic",
+            "config": {"workload": f"activation quantize, fp32 [{M}x{K}] -> tiled Q8_0 (cache-resident at this size: 10.6 MB)"},
+            "roofline": {"bound": "hbm", "kernel": "nh::quantize_kernel<true>", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n},
+        }
+
+    shapes = [(4096, K), (14336, K)]
+    ws = [q8_0.tile(q8_0.fill_weight_blocks(3 + i, n, k), n, k) for i, (n, k) in enumerate(shapes)]
+    outs = [torch.empty((M, n), dtype=torch.float32, device=x.device) for n, _ in shapes]
+    aq = q8_0.quantize_row_q8_0(x, tiled=True)
+
+    def fn():
+        for w, c, (n, k) in zip(ws, outs, shapes):
+            _lib.check("nh_q8_0_gemm_tiled", lib.nh_q8_0_gemm_tiled(w.data_ptr(), aq.data_ptr(), c.data_ptr(), M, n, k, stream))
+
+    ops = sum(2.0 * M * n * k for n, k in shapes)
+    wall, ksec, n_l = timed(2, fn, len(shapes))
+    ach = (ops / len(shapes)) / ksec / 1e12
+    return {
+        "metric": "Q8_0 prefill mat-mat TOP/s (int8 MFMA)", "value": round(ops / wall / 1e12, 1), "unit": "TOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "dtype": "int8 x int8 -> int32 block sums (MFMA), fp32 scale-accumulate", "data": "synthetic",
+        "config": {"workload": "prefill mat-mat, M=512 quantized activations x Q8_0 W [4096x4096] and [14336x4096] (two launches per step)"},
+        "roofline": {"bound": "mfma", "kernel": "nh::gemm_tiled_kernel<TM, DUMP=false>", "achieved": round(ach, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": round(ach / INT8_MFMA_PEAK_TOPS, 4), "traffic": None, "ops_per_launch": ops / len(shapes), "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n_l},
+    }
 
 
 def decode_step(tokens: int) -> dict:

@@ -13,7 +13,6 @@
 // tiles in exactly that order, so operands go from memory to the MFMA with one 16-byte load per lane and no
 // shuffle.  Result lanes: register i of lane l is C[m = 8*(i/4) + 4*(l/32) + i%4][n = l % 32].
 #include "q8_0_device.h"
-#include <type_traits>
 
 namespace nh {
 
@@ -151,255 +150,194 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const uint8_t* __res
 // The prefill kernel for the tiled layout.
 //
 // Both operands carry a scale per 32-quant block, so each 32x32x32 int8 MFMA result (1024 exact block sums, 16 per
-// lane) has to be converted and folded into the fp32 accumulator before the next block.  That makes the kernel
-// VALU-bound, not MFMA-bound: 16 conversions + 16 multiply-adds per lane per MFMA is 128 VALU cycles against 32
-// MFMA cycles on the same SIMD, so the design goal is to spend NOTHING else on the VALU:
-//   * the scale products f32(dA[m][b]) * f32(dW[n][b]) are formed on the matrix pipe too: one v_mfma_f32_32x32x8_f16
-//     whose A operand is the lane's four fp16 block scales as stored (row l%32, k = block within the group) and whose
-//     B operand is the weight row's four scales with all but block b masked off.  The product of two fp16 values is
-//     exact in fp32 (fp16 subnormals included), and it lands in the int8 MFMA's own accumulator layout, so the scales
-//     never need a conversion, a broadcast or a cross-lane move;
-//   * operands reach the waves through LDS: a workgroup copies whole 4352-byte macro-tiles (four blocks of 32 rows
-//     plus their scales) global -> registers -> LDS, double-buffered, one barrier per 128-quant group; waves read
-//     their 32x32 tiles back as conflict-free 16-byte-per-lane reads that already are MFMA operands.
-// Workgroup = 4 waves in a 2 x 2 arrangement, each wave TM x TN tiles of 32 x 32.
-template<int TM, int TN, bool DUMP>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums, int M, int N,
+// lane) has to be converted and folded into the fp32 accumulator before the next block: 16 conversions + 16
+// multiply-adds per lane per MFMA.  Measured on this part, a SIMD retires one wave64 VALU instruction per ~2.4 cycles
+// once it holds two or more waves (a lone wave issues one per ~5), and MFMA and VALU work does not overlap: a
+// (tile, block) costs 32 + 32 matrix-pipe cycles plus 32 x 2.4 VALU cycles, ~141 cycles against the 32 of the int8
+// MFMA alone.  That is the ceiling (~22 % of the int8 MFMA peak); the kernel is shaped to add as little as possible:
+//   * the scale products f32(dA[m][b]) * f32(dW[n][b]) are formed on the matrix pipe: one v_mfma_f32_32x32x8_f16 whose
+//     operands are the two blocks' fp16 scales as stored, each in the k = 0 slot ({d, 0, 0, 0}; lanes 32..63 supply
+//     the k = 4..7 slots = 0).  The product of two fp16 values is exact in fp32 (fp16 subnormals included) and lands
+//     in the int8 MFMA's own accumulator layout: no conversion, broadcast or cross-lane move of a scale, ever;
+//   * only the operand that is shared goes through LDS.  A workgroup is four waves; wave w owns weight strip
+//     4*blockIdx.x + w and loads its tiles straight from global memory into registers (one coalesced 16-byte-per-lane
+//     load per tile, already an MFMA operand, a whole 128-quant group ahead of use); all four waves share the same
+//     TM activation strips, copied global -> LDS one group ahead (double-buffered, one barrier per group, the copy
+//     spread over the four waves) and read back as conflict-free 16-byte-per-lane operand images plus one half-word
+//     read per scale;
+//   * latency is hidden by occupancy, not by a software pipeline: one result-register set per tile keeps the kernel
+//     at <= 128 VGPRs, four workgroups per CU, four waves per SIMD.  (A two-result-set, software-pipelined variant
+//     at two waves per SIMD measured 8 % slower: with so few waves the SIMD falls back to the lone-wave issue rate
+//     whenever one of them waits.)
+template<int TM, bool DUMP>
+__global__ __launch_bounds__(256, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums, int M, int N,
 	int groups) {
-	constexpr int SA		  = 2 * TM; // A strips per workgroup
-	constexpr int SW		  = 2 * TN; // W strips per workgroup
-	constexpr int STRIPS	  = SA + SW;
-	constexpr int DATA_BYTES  = STRIPS * MACRO_BYTES;
-	constexpr int STAGE_BYTES = DATA_BYTES + 16; // + 16 zero bytes: what lanes 32..63 feed the scale MFMA (k = 4..7)
-	extern __shared__ __align__(16) uint8_t lds[]; // [2][STAGE_BYTES]
-	if (threadIdx.x < 8) {
-		*reinterpret_cast<uint32_t*>(lds + (threadIdx.x >> 2) * STAGE_BYTES + DATA_BYTES + 4 * (threadIdx.x & 3)) = 0u; // made visible by the first barrier below
-	}
-
+	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
+	constexpr int STAGE_BYTES = DATA_BYTES + 16;
+	__shared__ __align__(16) uint8_t lds[2 * STAGE_BYTES];
 	typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 	typedef float v16f __attribute__((ext_vector_type(16)));
 
 	const int tid	   = threadIdx.x;
 	const int lane	   = tid & 63;
 	const int wave	   = __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int wm	   = wave >> 1;
-	const int wn	   = wave & 1;
 	const int half	   = lane >> 5;
 	const int m_strips = (M + 31) / 32;
 	const int n_strips = (N + 31) / 32;
-	const int ms0	   = blockIdx.y * SA; // first A strip of the workgroup
-	const int ns0	   = blockIdx.x * SW;
-
-	// Global -> LDS copy: whole macro-tiles, one per wave at a time (wave w moves strips w, w+4, ...).  4352 bytes are
-	// 64 lanes x (4 x 16 B + 4 B): every lane is live in every load, so the copy needs no predicate and no zero fill.
-	// Strips past the matrix edge are clamped to the last real one: their products are computed and never stored.
-	constexpr int COPIES = (STRIPS + 3) / 4;
-	const uint8_t* src[COPIES];
-#pragma unroll
-	for (int c = 0; c < COPIES; ++c) {
-		const int strip = min(wave + 4 * c, STRIPS - 1); // the last round may repeat a strip: same bytes, same place
-		const uint8_t* base;
-		if (strip < SA) {
-			base = A + macro_offset(min(ms0 + strip, m_strips - 1), 0, groups);
-		} else {
-			base = W + macro_offset(min(ns0 + strip - SA, n_strips - 1), 0, groups);
-		}
-		src[c] = base;
+	const int ms0	   = blockIdx.y * TM;
+	const int ns	   = blockIdx.x * 4 + wave;
+	if (tid < 8) {
+		*reinterpret_cast<uint32_t*>(lds + (tid >> 2) * STAGE_BYTES + DATA_BYTES + 4 * (tid & 3)) = 0u;
 	}
-	struct copy_regs {
-		v4i q[COPIES][4];
-		uint32_t d[COPIES];
+	const uint8_t* w_src = W + macro_offset(min(ns, n_strips - 1), 0, groups);
+	struct w_regs {
+		v4i q[GROUP_BLOCKS];
+		v2u d;
 	};
-	auto fetch = [&](int g, copy_regs& r) {
+	auto fetch_w = [&](int g, w_regs& r) {
+		const uint8_t* p = w_src + static_cast<int64_t>(g) * MACRO_BYTES;
 #pragma unroll
-		for (int c = 0; c < COPIES; ++c) {
-			const uint8_t* p = src[c] + static_cast<int64_t>(g) * MACRO_BYTES;
+		for (int k = 0; k < GROUP_BLOCKS; ++k) {
+			r.q[k] = *reinterpret_cast<const v4i*>(p + k * TILE_BYTES + 16 * lane);
+		}
+		r.d = *reinterpret_cast<const v2u*>(p + MACRO_D_OFFSET + 8 * (lane & 31));
+	};
+	// activations: global -> registers -> LDS, shared out over the four waves: wave w moves tiles TM*w .. TM*w+TM-1 of the
+	// TM*4 tiles of a group, waves 0..TM-1 also the 256-byte scale table of strip w
+	const uint8_t* a_src[TM];
+	int a_dst[TM];
 #pragma unroll
-			for (int k = 0; k < 4; ++k) {
-				r.q[c][k] = *reinterpret_cast<const v4i*>(p + k * TILE_BYTES + 16 * lane);
-			}
-			r.d[c] = *reinterpret_cast<const uint32_t*>(p + MACRO_D_OFFSET + 4 * lane);
+	for (int j = 0; j < TM; ++j) {
+		const int u = TM * wave + j;
+		a_src[j]	= A + macro_offset(min(ms0 + u / 4, m_strips - 1), 0, groups) + (u % 4) * TILE_BYTES + 16 * lane;
+		a_dst[j]	= (u / 4) * MACRO_BYTES + (u % 4) * TILE_BYTES + 16 * lane;
+	}
+	const bool sc_copier   = wave < TM;
+	const uint8_t* sc_src = A + macro_offset(min(ms0 + min(wave, TM - 1), m_strips - 1), 0, groups) + MACRO_D_OFFSET + 4 * lane;
+	const int sc_dst	   = min(wave, TM - 1) * MACRO_BYTES + MACRO_D_OFFSET + 4 * lane;
+	struct a_regs {
+		v4i q[TM];
+		uint32_t d;
+	};
+	auto fetch_a = [&](int g, a_regs& r) {
+#pragma unroll
+		for (int j = 0; j < TM; ++j) {
+			r.q[j] = *reinterpret_cast<const v4i*>(a_src[j] + static_cast<int64_t>(g) * MACRO_BYTES);
+		}
+		if (sc_copier) {
+			r.d = *reinterpret_cast<const uint32_t*>(sc_src + static_cast<int64_t>(g) * MACRO_BYTES);
 		}
 	};
-	auto stash = [&](int stage, const copy_regs& r) {
+	auto stash_a = [&](int stage, const a_regs& r) {
+		uint8_t* p = lds + stage * STAGE_BYTES;
 #pragma unroll
-		for (int c = 0; c < COPIES; ++c) {
-			uint8_t* p = lds + stage * STAGE_BYTES + min(wave + 4 * c, STRIPS - 1) * MACRO_BYTES;
-#pragma unroll
-			for (int k = 0; k < 4; ++k) {
-				*reinterpret_cast<v4i*>(p + k * TILE_BYTES + 16 * lane) = r.q[c][k];
-			}
-			*reinterpret_cast<uint32_t*>(p + MACRO_D_OFFSET + 4 * lane) = r.d[c];
+		for (int j = 0; j < TM; ++j) {
+			*reinterpret_cast<v4i*>(p + a_dst[j]) = r.q[j];
+		}
+		if (sc_copier) {
+			*reinterpret_cast<uint32_t*>(p + sc_dst) = r.d;
 		}
 	};
-
-	v16f acc[TM][TN];
+	v16f acc[TM];
 #pragma unroll
 	for (int i = 0; i < TM; ++i) {
-#pragma unroll
-		for (int j = 0; j < TN; ++j) {
-			acc[i][j] = v16f{ 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-		}
+		acc[i] = v16f{ 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
 	}
+	const int a_sc_rel = half ? DATA_BYTES : MACRO_D_OFFSET + 8 * (lane & 31);
 
-	// One block's worth of matrix-pipe work for this wave: TM*TN int8 MFMAs (block sums) and as many f16 MFMAs (scale
-	// products), results in sv / pv.  Everything an MFMA needs comes out of LDS in its final form, so this half costs
-	// the VALU nothing: the quants as 16-byte operand images, the scales as single zero-extended half-word reads
-	// ({d, 0, 0, 0} in the k = 0..3 slots; lanes 32..63, the k = 4..7 slots, read the stage's zero bytes instead).
-	// The compiler fence pins the LDS reads -- and with them the MFMAs that depend on them -- behind the previous
-	// pipeline step; without it every MFMA of a group is hoisted to the front and the result registers overflow.
-	const int sc_rel = half ? DATA_BYTES : MACRO_D_OFFSET + 8 * (lane & 31); // + strip*MACRO_BYTES for live lanes, see below
-	auto issue = [&](const uint8_t* stage, auto t_const, v16i(&sv)[TM][TN], v16f(&pv)[TM][TN]) {
-		constexpr int t = decltype(t_const)::value;
-		asm volatile("" ::: "memory");
-		v4i a[TM], w[TN];
-		v2u a_sc[TM], w_sc[TN];
-#pragma unroll
-		for (int i = 0; i < TM; ++i) {
-			const int strip = wm * TM + i;
-			a[i]			= *reinterpret_cast<const v4i*>(stage + strip * MACRO_BYTES + t * TILE_BYTES + 16 * lane);
-			a_sc[i]			= v2u{ *reinterpret_cast<const uint16_t*>(stage + (half ? 0 : strip * MACRO_BYTES) + sc_rel + 2 * t), 0u };
+	w_regs wa, wb;
+	a_regs pre;
+	fetch_w(0, wa);
+	fetch_a(0, pre);
+	stash_a(0, pre);
+	__syncthreads();
+	auto trip = [&](int g, w_regs& cur, w_regs& nxt) {
+		const bool more = g + 1 < groups;
+		if (more) {
+			fetch_w(g + 1, nxt);
+			fetch_a(g + 1, pre);
 		}
-#pragma unroll
-		for (int j = 0; j < TN; ++j) {
-			const int strip = SA + wn * TN + j;
-			w[j]			= *reinterpret_cast<const v4i*>(stage + strip * MACRO_BYTES + t * TILE_BYTES + 16 * lane);
-			w_sc[j]			= v2u{ *reinterpret_cast<const uint16_t*>(stage + (half ? 0 : strip * MACRO_BYTES) + sc_rel + 2 * t), 0u };
+		if (half) {
+			cur.d = v2u{ 0u, 0u };
 		}
+		const uint8_t* stage = lds + (g & 1) * STAGE_BYTES;
 #pragma unroll
-		for (int j = 0; j < TN; ++j) {
+		for (int t = 0; t < GROUP_BLOCKS; ++t) {
+			const uint32_t wd = (t < 2) ? cur.d.x : cur.d.y;
+			const v2u w_sc	  = v2u{ (t & 1) ? (wd >> 16) : (wd & 0xFFFFu), 0u };
 #pragma unroll
 			for (int i = 0; i < TM; ++i) {
-				const v16i zi = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-				const v16f zf = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-				sv[i][j]	  = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], w[j], zi, 0, 0, 0);
-				if constexpr (!DUMP) {
-					pv[i][j] = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, a_sc[i]), __builtin_bit_cast(v4h, w_sc[j]), zf, 0, 0, 0);
-				}
-			}
-		}
-	};
-	// The VALU half: convert the block sums and fold them into the accumulators with their scale products.
-	auto fold = [&](int block, const v16i(&sv)[TM][TN], const v16f(&pv)[TM][TN]) {
-#pragma unroll
-		for (int i = 0; i < TM; ++i) {
-#pragma unroll
-			for (int j = 0; j < TN; ++j) {
+				asm volatile("" ::: "memory");
+				const v4i a		= *reinterpret_cast<const v4i*>(stage + i * MACRO_BYTES + t * TILE_BYTES + 16 * lane);
+				const v2u a_sc	= v2u{ *reinterpret_cast<const uint16_t*>(stage + (half ? 0 : i * MACRO_BYTES) + a_sc_rel + 2 * t), 0u };
+				const v16i zi	= { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+				const v16f zf	= { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+				const v16i sv	= __builtin_amdgcn_mfma_i32_32x32x32_i8(a, cur.q[t], zi, 0, 0, 0);
 				if constexpr (DUMP) {
-					const int n = (ns0 + wn * TN + j) * 32 + (lane & 31);
+					const int n = ns * 32 + (lane & 31);
 #pragma unroll
 					for (int e = 0; e < 16; ++e) {
-						const int m = (ms0 + wm * TM + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+						const int m = (ms0 + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 						if (m < M && n < N) {
-							sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + block] = sv[i][j][e];
+							sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + g * GROUP_BLOCKS + t] = sv[e];
 						}
 					}
 				} else {
+					const v16f pv = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, a_sc), __builtin_bit_cast(v4h, w_sc), zf, 0, 0, 0);
 #pragma unroll
 					for (int e = 0; e < 16; ++e) {
-						acc[i][j][e] = fmaf(static_cast<float>(sv[i][j][e]), pv[i][j][e], acc[i][j][e]);
+						acc[i][e] = fmaf(static_cast<float>(sv[e]), pv[e], acc[i][e]);
 					}
-					// pins this fold in program order (no instruction is emitted): the arithmetic above has no side effect, and
-					// left free it is sunk to the end of the loop, behind every MFMA of the group
-					asm volatile("" : "+v"(acc[i][j]));
+					asm volatile("" : "+v"(acc[i]));
 				}
 			}
 		}
+		if (more) {
+			stash_a((g + 1) & 1, pre);
+		}
+		__syncthreads();
 	};
-	using t0 = std::integral_constant<int, 0>;
-	using t1 = std::integral_constant<int, 1>;
-	using t2 = std::integral_constant<int, 2>;
-	using t3 = std::integral_constant<int, 3>;
-
-	copy_regs pre;
-	fetch(0, pre);
-	stash(0, pre);
-	__syncthreads();
-
-	// Software pipeline, one block deep: while the VALU folds block b, the matrix pipe already works on block b+1
-	// (two register sets, s0/p0 and s1/p1).  The scheduling fences keep the compiler from hoisting more than that:
-	// left alone it moves every MFMA of a group to the front and the result registers overflow the file.
-	v16i s0[TM][TN], s1[TM][TN];
-	v16f p0[TM][TN], p1[TM][TN];
-	issue(lds, t0{}, s0, p0);
-	__builtin_amdgcn_sched_barrier(0);
-	for (int g = 0; g < groups; ++g) {
-		const bool more = g + 1 < groups;
-		if (more) {
-			fetch(g + 1, pre); // global loads in flight across the next three folds
+	for (int g = 0; g < groups; g += 2) {
+		trip(g, wa, wb);
+		if (g + 1 < groups) {
+			trip(g + 1, wb, wa);
 		}
-		const uint8_t* stage = lds + (g & 1) * STAGE_BYTES;
-		const int b0		 = g * GROUP_BLOCKS;
-		issue(stage, t1{}, s1, p1);
-		fold(b0 + 0, s0, p0);
-		__builtin_amdgcn_sched_barrier(0);
-		issue(stage, t2{}, s0, p0);
-		fold(b0 + 1, s1, p1);
-		__builtin_amdgcn_sched_barrier(0);
-		issue(stage, t3{}, s1, p1);
-		fold(b0 + 2, s0, p0);
-		__builtin_amdgcn_sched_barrier(0);
-		if (more) {
-			// the other stage was last read during the previous trip, and a barrier has passed since
-			stash((g + 1) & 1, pre);
-		}
-		__syncthreads(); // every wave is done reading this stage's tiles (all four issues are behind it) and the next stage is complete
-		if (more) {
-			const uint8_t* next = lds + ((g + 1) & 1) * STAGE_BYTES;
-			issue(next, t0{}, s0, p0);
-		}
-		fold(b0 + 3, s1, p1);
-		__builtin_amdgcn_sched_barrier(0);
 	}
-
 	if constexpr (!DUMP) {
+		const int n = ns * 32 + (lane & 31);
 #pragma unroll
 		for (int i = 0; i < TM; ++i) {
 #pragma unroll
-			for (int j = 0; j < TN; ++j) {
-				const int n = (ns0 + wn * TN + j) * 32 + (lane & 31);
-#pragma unroll
-				for (int e = 0; e < 16; ++e) {
-					const int m = (ms0 + wm * TM + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-					if (m < M && n < N) {
-						C[static_cast<int64_t>(m) * N + n] = acc[i][j][e];
-					}
+			for (int e = 0; e < 16; ++e) {
+				const int m = (ms0 + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+				if (m < M && n < N) {
+					C[static_cast<int64_t>(m) * N + n] = acc[i][e];
 				}
 			}
 		}
 	}
 }
 
-template<int TM, int TN> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int k, hipStream_t s) {
+template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int k, hipStream_t s) {
 	const int groups   = k / GROUP_K;
 	const int m_strips = (m + 31) / 32, n_strips = (n + 31) / 32;
-	const dim3 grid(static_cast<unsigned>((n_strips + 2 * TN - 1) / (2 * TN)), static_cast<unsigned>((m_strips + 2 * TM - 1) / (2 * TM)));
-	const size_t shmem = 2 * (static_cast<size_t>(2 * TM + 2 * TN) * MACRO_BYTES + 16);
-	hipError_t e	   = hipSuccess;
-	if (shmem > 64 * 1024) { // more than the default dynamic-LDS limit: opt in once per kernel
-		static bool raised_plain = false, raised_dump = false;
-		bool& raised = sums ? raised_dump : raised_plain;
-		if (!raised) {
-			e = sums ? hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiled_kernel<TM, TN, true>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shmem))
-					 : hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiled_kernel<TM, TN, false>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shmem));
-			if (e != hipSuccess) {
-				return e;
-			}
-			raised = true;
-		}
-	}
+	const dim3 grid(static_cast<unsigned>((n_strips + 3) / 4), static_cast<unsigned>((m_strips + TM - 1) / TM));
 	if (sums) {
-		gemm_tiled_kernel<TM, TN, true><<<grid, dim3(256), shmem, s>>>(w, a, C, sums, m, n, groups);
+		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, sums, m, n, groups);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, TN, false>, grid, dim3(256), shmem, s, w, a, C, sums, m, n, groups);
+	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false>, grid, dim3(256), 0, s, w, a, C, sums, m, n, groups);
 }
 
-// Tile choice.  The kernel is bound by VALU issue, and one wave alone issues a VALU instruction only every ~5 cycles
-// (two or more per SIMD reach ~2.4), so occupancy matters more than operand reuse: 64 x 64 workgroup tiles (TM = TN = 1,
-// ~120 VGPRs, 35 KB LDS: four workgroups per CU) measured faster than 64 x 128 at every prefill shape tried.
+// Tile choice.  One wave alone issues a VALU instruction only every ~5 cycles (two or more per SIMD reach ~2.4), so
+// the grid must give every SIMD at least two waves: 64-row workgroup tiles (half the LDS and L2 traffic per MFMA) when
+// that still leaves >= 512 workgroups, 32-row tiles otherwise.
 static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int k, hipStream_t s) {
-	return launch_gemm_tiled_t<1, 1>(w, a, C, sums, m, n, k, s);
+	const int64_t ms = (m + 31) / 32, ns4 = ((n + 31) / 32 + 3) / 4;
+	if (((ms + 1) / 2) * ns4 >= 1024) {
+		return launch_gemm_tiled_t<2>(w, a, C, sums, m, n, k, s);
+	}
+	return launch_gemm_tiled_t<1>(w, a, C, sums, m, n, k, s);
 }
 
 __global__ void zero_c_kernel(float* __restrict__ c, int64_t n) {
