@@ -60,7 +60,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
     ap.add_argument("--calibration-copies", type=int, default=0, help="run this many plain 64 MiB device copies first (a known-size kernel to scale hardware byte counters by)")
-    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize"], default="ffn_decode",
+    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode-step leg (8 GB of weights)")
@@ -216,8 +216,9 @@ INT8_MFMA_PEAK_TOPS = 5033.0  # MI355X published dense int8 matrix rate
 
 
 def side_workload(kind: str, steps: int, warmup: int) -> dict:
-    """One JSON line for the prefill mat-mat (BASELINE config 3: M=512, W [4096x4096] and [14336x4096]) or for the
-    stand-alone activation quantize (M=512, K=4096), each against the roofline that bounds it."""
+    """One JSON line for the prefill mat-mat (BASELINE config 3: M=512, W [4096x4096] and [14336x4096]), for the
+    stand-alone activation quantize (M=512, K=4096) or for the token-embedding lookup (512 tokens), each against
+    the roofline that bounds it."""
     import torch
 
     from nihilus_amd import _lib, q8_0
@@ -259,6 +260,26 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
             "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "dtype": "fp32 -> int8 + fp16 scale", "data": "synthetic",
             "config": {"workload": f"activation quantize, fp32 [{M}x{K}] -> tiled Q8_0 (cache-resident at this size: 10.6 MB)"},
             "roofline": {"bound": "hbm", "kernel": "nh::quantize_kernel<true>", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n},
+        }
+
+    if kind == "get_rows":
+        n_rows = 128256  # LLaMA-3 vocabulary; token_embd.weight [4096 x 128256] Q8_0 = 558 MB, rows picked at random
+        table = q8_0.tile(q8_0.fill_weight_blocks(9, n_rows, K), n_rows, K)
+        ids = torch.randint(0, n_rows, (M,), dtype=torch.int32, device=x.device)
+        out = torch.empty((M, K), dtype=torch.float32, device=x.device)
+        nbytes = M * (K // 32) * 34 + 4 * M * K + 4 * M
+
+        def fn():
+            _lib.check("nh_q8_0_get_rows_tiled", lib.nh_q8_0_get_rows_tiled(table.data_ptr(), ids.data_ptr(), out.data_ptr(), None, M, n_rows, K, stream))
+
+        wall, ksec, n = timed(3, fn, 1)
+        ach = nbytes / ksec / 1e9
+        return {
+            "metric": "Q8_0 token-embedding get_rows GB/s", "value": round(nbytes / wall / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "dtype": "int8 x fp16 scale -> fp32", "data": "synthetic",
+            "config": {"workload": f"token-embedding lookup, {M} random rows of a tiled Q8_0 table [{n_rows}x{K}] -> fp32 [{M}x{K}]"},
+            "roofline": {"bound": "hbm", "kernel": "nh::get_rows_kernel<TILED=true>", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n},
         }
 

@@ -156,6 +156,23 @@ namespace nihilus {
 		static_assert(output_dims[3] == input_01_dims[3] || output_dims[3] == input_02_dims[3], "mul_mat: batch dim 3 must match an input");
 	};
 
+	// get_rows: out[ne0 = K, ne1 = tokens] = rows of table[K, n_rows] picked by ids[tokens]; the reference's shape rules
+	// (common/kernel_traits.hpp:646-665).
+	template<typename config_type, typename dims_type_new, typename output_type_new, typename input_01_type_new, typename input_02_type_new>
+	struct kernel_traits_old<config_type, dims_type_new, kernel_types::get_rows, output_type_new, input_01_type_new, input_02_type_new> : public dims_type_new {
+		using input_01_type					= input_01_type_new;
+		using input_02_type					= input_02_type_new;
+		using output_type					= output_type_new;
+		using dims_type						= dims_type_new;
+		static constexpr auto input_01_dims = input_01_type::get_array();
+		static constexpr auto input_02_dims = input_02_type::get_array();
+		static constexpr auto output_dims	= dims_type::get_array();
+		static_assert(input_02_dims[0] == output_dims[1], "get_rows: one index per output row");
+		static_assert(input_02_dims[1] == 1 && input_02_dims[2] == 1 && input_02_dims[3] == 1, "get_rows: indices are one-dimensional");
+		static_assert(output_dims[0] == input_01_dims[0], "get_rows: output row length must equal the embedding length");
+		static_assert(output_dims[2] == 1 && output_dims[3] == 1, "get_rows: output is two-dimensional");
+	};
+
 	// throw, or log and std::exit(-1), chosen by the config at compile time
 	template<bool exceptions> struct nihilus_exception_impl {
 		[[noreturn]] static void impl(std::string_view error_type, std::string_view detail, const std::source_location& where) {
@@ -238,11 +255,46 @@ namespace nihilus {
 		}
 	};
 
+	// get_rows (token embeddings), both phases: out[t][:] = dequantized row ids[t] of the embedding table.  The table
+	// operand holds the device copy of token_embd.weight, tiled (table_is_tiled) or as the packed blocks of the file.
+	// eval_time looks up one token, prompt_eval_time the output's runtime sequence length; both index by the id (the
+	// reference's CUDA eval-time kernel, cuda/cuda_12.hpp:691-722, dequantizes row 0 whatever the id).
+	template<typename config_type, typename core_traits_type, processing_phases processing_phase>
+	struct kernel_dispatcher_impl<config_type, core_traits_type, device_types::gpu, 5, kernel_types::get_rows, processing_phase, core_traits_type, float, block_q8_0<half>,
+		int32_t> {
+		using input_type01			   = typename core_traits_type::input_01_type;
+		static constexpr uint64_t ne00 = input_type01::get_array()[0]; // embedding length
+		static constexpr uint64_t ne01 = input_type01::get_array()[1]; // vocabulary size
+
+		static void impl(core_traits_type& output, const void* table, bool table_is_tiled, const int32_t* token_ids, void* stream = nullptr) {
+			uint64_t tokens = 1;
+			if constexpr (processing_phase == processing_phases::prompt_eval_time) {
+				tokens = output.get_seq_length_dim();
+				if (tokens == 0) {
+					return;
+				}
+			}
+			const auto fn = table_is_tiled ? nh_q8_0_get_rows_tiled : nh_q8_0_get_rows;
+			amd_detail::check<config_type>(fn(table, token_ids, output.template get_data<float>(), nullptr, static_cast<int64_t>(tokens), ne01, ne00, stream), "get_rows");
+			if constexpr (config_type::synchronous) {
+				amd_detail::check<config_type>(nh_stream_sync(stream), "stream sync");
+			}
+		}
+	};
+
 	// Caller-side helper: picks the specialisation from the config, as kernel_dispatcher does for the mega kernels
 	// (infra/monolithic_dispatcher.hpp:41-63).
 	template<typename config_type, processing_phases processing_phase, typename mul_mat_traits_type> struct mul_mat_dispatcher {
 		using impl_type = kernel_dispatcher_impl<config_type, mul_mat_traits_type, config_type::device_type, arch_index<config_type::device_type>, kernel_types::mul_mat,
 			processing_phase, mul_mat_traits_type, float, block_q8_0<half>, block_q8_0<half>>;
+		template<typename... arg_types> static void impl(arg_types&&... args) {
+			impl_type::impl(std::forward<arg_types>(args)...);
+		}
+	};
+
+	template<typename config_type, processing_phases processing_phase, typename get_rows_traits_type> struct get_rows_dispatcher {
+		using impl_type = kernel_dispatcher_impl<config_type, get_rows_traits_type, config_type::device_type, arch_index<config_type::device_type>, kernel_types::get_rows,
+			processing_phase, get_rows_traits_type, float, block_q8_0<half>, int32_t>;
 		template<typename... arg_types> static void impl(arg_types&&... args) {
 			impl_type::impl(std::forward<arg_types>(args)...);
 		}

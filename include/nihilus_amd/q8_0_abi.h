@@ -89,6 +89,18 @@ int64_t nh_q8_0_tiled_bytes(int64_t rows, int64_t K);
 int nh_q8_0_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, void* stream);
 int nh_q8_0_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, void* stream);
 
+/* Token-embedding lookup (get_rows) ------------------------------------------------------------- */
+
+/* out[t][j] = f32(d[ids[t]][j/32]) * f32(qs[ids[t]][j]),  t < n_tokens, j < K: one fp32 multiply per element,
+ * bit-exact against the CPU.  Replaces the reference's live token_embeddings kernels, both phases
+ * (cpu/avx_2.hpp:40-66, :68-140; per-op form :1241-1294; cuda/cuda_12.hpp:560-601, and :691-722 whose missing
+ * token index is not reproduced).  W: the [n_rows x K] embedding matrix, device, blocks or tiled layout;
+ * ids: int32 [n_tokens], device (global_input_types::inp_tokens); out: fp32 [n_tokens][K], device.
+ * The reference reads whatever row an id names; here an id outside [0, n_rows) yields a row of zeros and, if
+ * invalid_count is not NULL, adds one to that device int32 (the caller zeroes it). K % 32 == 0 (tiled: % 128). */
+int nh_q8_0_get_rows(const void* W_blocks, const int32_t* ids, float* out, int32_t* invalid_count, int64_t n_tokens, int64_t n_rows, int64_t K, void* stream);
+int nh_q8_0_get_rows_tiled(const void* W_tiled, const int32_t* ids, float* out, int32_t* invalid_count, int64_t n_tokens, int64_t n_rows, int64_t K, void* stream);
+
 /* Mat-vec (decode, eval_time) ------------------------------------------------------------------- */
 
 /* y[n] = sum_b f32(dW[n][b]) * f32(dx[b]) * sum_{j<32} W.qs[n][b][j] * x.qs[b][j]
@@ -143,7 +155,7 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 
 /* Per-kernel timing (instrumentation) ----------------------------------------------------------- */
 
-/* kernel_kind: 0 = quantize, 1 = mat-vec, 2 = mat-mat.  Between begin and end every launch of that kind (up to
+/* kernel_kind: 0 = quantize, 1 = mat-vec, 2 = mat-mat, 3 = get_rows.  Between begin and end every launch of that kind (up to
  * max_launches) records GPU timestamps at the kernel's own start and end.  nh_profile_end waits for them and
  * returns the summed, smallest and largest kernel durations in milliseconds.  Process-wide; not for concurrent use. */
 int nh_profile_begin(int kernel_kind, int64_t max_launches);

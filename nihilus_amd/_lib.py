@@ -29,6 +29,8 @@ SIGNATURES = {
     "nh_q8_0_tiled_bytes": (_i64, [_i64, _i64]),
     "nh_q8_0_tile": (_int, [_vp, _vp, _i64, _i64, _vp]),
     "nh_q8_0_untile": (_int, [_vp, _vp, _i64, _i64, _vp]),
+    "nh_q8_0_get_rows": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "nh_q8_0_get_rows_tiled": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "nh_q8_0_gemv": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "nh_q8_0_gemv_tiled": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "nh_q8_0_gemv_tiled_f32": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),

@@ -238,6 +238,25 @@ int nh_q8_0_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, voi
 	return from_hip(nh::launch_untile(tiled, blocks, rows, K, as_stream(stream)));
 }
 
+static int get_rows_common(const void* W, const int32_t* ids, float* out, int32_t* invalid_count, int64_t n_tokens, int64_t n_rows, int64_t K, bool tiled, void* stream) {
+	NH_TRY(check_shape(n_rows, n_tokens, K, tiled));
+	if (n_tokens == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(ids && out && (W || n_rows == 0), NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(W) && aligned16(out) && reinterpret_cast<uintptr_t>(ids) % 4 == 0 && reinterpret_cast<uintptr_t>(invalid_count) % 4 == 0, NH_ERR_ALIGNMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_get_rows(W, ids, out, invalid_count, n_tokens, n_rows, K, tiled, as_stream(stream)));
+}
+
+int nh_q8_0_get_rows(const void* W_blocks, const int32_t* ids, float* out, int32_t* invalid_count, int64_t n_tokens, int64_t n_rows, int64_t K, void* stream) {
+	return get_rows_common(W_blocks, ids, out, invalid_count, n_tokens, n_rows, K, false, stream);
+}
+
+int nh_q8_0_get_rows_tiled(const void* W_tiled, const int32_t* ids, float* out, int32_t* invalid_count, int64_t n_tokens, int64_t n_rows, int64_t K, void* stream) {
+	return get_rows_common(W_tiled, ids, out, invalid_count, n_tokens, n_rows, K, true, stream);
+}
+
 static int gemv_common(const void* W, const void* xq, float* y, int64_t N, int64_t K, bool tiled, void* stream) {
 	NH_TRY(check_shape(N, 0, K, tiled));
 	NH_REQUIRE(tiled || K <= MAX_K_BLOCKS_GEMV, NH_ERR_TOO_LARGE);

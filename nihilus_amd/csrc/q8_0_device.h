@@ -80,7 +80,7 @@ __device__ __host__ __forceinline__ int64_t macro_offset(int64_t strip, int64_t 
 
 // ---- per-kernel timing (opt-in instrumentation, see q8_0_profile.hip) ----
 
-enum kernel_kind : int { KIND_QUANTIZE = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_COUNT = 3 };
+enum kernel_kind : int { KIND_QUANTIZE = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GET_ROWS = 3, KIND_COUNT = 4 };
 
 // When timing is on for `kind` and the event pool has room, hands out an event pair for the next launch.
 bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop);
@@ -103,6 +103,7 @@ inline hipError_t launch_kernel(int kind, Kernel kernel, dim3 grid, dim3 block, 
 hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s);
 hipError_t launch_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, hipStream_t s);
 hipError_t launch_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, hipStream_t s);
+hipError_t launch_get_rows(const void* W, const int32_t* ids, float* out, int32_t* invalid, int64_t n_tokens, int64_t n_rows, int64_t K, bool tiled, hipStream_t s);
 hipError_t launch_fill_weights(void* blocks, uint64_t seed, int64_t first_block, int64_t n_blocks, hipStream_t s);
 hipError_t launch_fill_activations(float* x, uint64_t seed, int64_t count, hipStream_t s);
 // sums == nullptr: production; otherwise the same kernel diverts the per-block int32 sums to `sums` and leaves y alone.

@@ -70,6 +70,21 @@ def untile(tiled: torch.Tensor, rows: int, k: int) -> torch.Tensor:
     return out
 
 
+def get_rows(w: torch.Tensor, ids: torch.Tensor, n_rows: int, k: int, tiled: bool, count_invalid: bool = False):
+    """Token-embedding lookup: fp32 [n_tokens, k] = dequantized rows `ids` of the Q8_0 matrix w (blocks or tiled).
+
+    With count_invalid the number of ids outside [0, n_rows) comes back as a second value (their rows are zero)."""
+    w, ids = _dev(w, torch.uint8, "w"), _dev(ids, torch.int32, "ids")
+    if w.numel() != (tiled_bytes(n_rows, k) if tiled else blocks_bytes(n_rows, k)):
+        raise ValueError("w has the wrong size for n_rows x k")
+    n_tokens = ids.numel()
+    out = torch.empty((n_tokens, k), dtype=torch.float32, device=w.device)
+    bad = torch.zeros(1, dtype=torch.int32, device=w.device) if count_invalid else None
+    fn = "nh_q8_0_get_rows_tiled" if tiled else "nh_q8_0_get_rows"
+    _lib.check(fn, getattr(_lib.lib(), fn)(w.data_ptr(), ids.data_ptr(), out.data_ptr(), bad.data_ptr() if count_invalid else None, n_tokens, n_rows, k, _stream()))
+    return (out, int(bad.item())) if count_invalid else out
+
+
 def gemv(w: torch.Tensor, xq_blocks: torch.Tensor, n: int, k: int, tiled: bool) -> torch.Tensor:
     w, xq_blocks = _dev(w, torch.uint8, "w"), _dev(xq_blocks, torch.uint8, "xq_blocks")
     if w.numel() != (tiled_bytes(n, k) if tiled else blocks_bytes(n, k)) or xq_blocks.numel() != blocks_bytes(1, k):

@@ -51,6 +51,7 @@ _a_fp16_to_fp32 = _sig(_a, "nha_fp16_to_fp32", C.c_float, C.c_uint16)
 _a_fp32_to_fp16 = _sig(_a, "nha_fp32_to_fp16", C.c_uint16, C.c_float)
 _q8_bytes = _sig(_o, "nho_q8_0_bytes", _i64, _i64, _i64)
 _dequant = _sig(_o, "nho_dequantize_row_q8_0", None, _vp, _vp, _i64)
+_get_rows = _sig(_o, "nho_get_rows_q8_0", _i64, _vp, _vp, _vp, _i64, _i64, _i64)
 _quant_rows = _sig(_o, "nho_quantize_rows_q8_0", None, _vp, _vp, _i64, _i64)
 _a_quant_rows = _sig(_a, "nha_quantize_rows_q8_0", None, _vp, _vp, _i64, _i64)
 _sums_gemv = _sig(_o, "nho_block_sums_gemv", None, _vp, _vp, _vp, _i64, _i64)
@@ -131,6 +132,15 @@ def dequantize_row(blocks: np.ndarray, k: int) -> np.ndarray:
     b = _u8(blocks)
     _dequant(_ptr(b), _ptr(y), k)
     return y
+
+
+def get_rows(blocks: np.ndarray, ids: np.ndarray, n_rows: int, k: int):
+    """Token-embedding lookup on a [n_rows, k] block matrix; returns (fp32 [n_tokens, k], number of out-of-range ids)."""
+    b = _u8(blocks)
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    out = np.empty((ids.size, k), dtype=np.float32)
+    bad = _get_rows(_ptr(b), _ptr(ids), _ptr(out), ids.size, n_rows, k)
+    return out, int(bad)
 
 
 # ---------------------------------------------------------------- quantize

@@ -22,6 +22,11 @@
  *                                        even, trailing k%32 ignored) and an independent numpy
  *                                        evaluation.  No reference-held vector exists: the
  *                                        reference has no test of this function.
+ *   nho_dequantize_row / nho_get_rows    independent numpy evaluation (numpy's own float16), real ggml blocks from
+ *                                        the reference's dumps used as an embedding table, a table whose row r
+ *                                        decodes to the constant r (index order), out-of-range ids.  The
+ *                                        reference's dump of this op's output (inp_embd) covers a vocabulary row
+ *                                        whose bytes are not in the dumps, so it cannot be replayed end to end.
  *   nho_block_sum_i32                    int64 brute force; extreme blocks (+-127 -> +-516128).
  *   nho_vec_dot_* / gemv / gemm          float64 evaluation (<= ~1e-6 rel), d == 1 gives exact
  *                                        integers, tiny hand-checkable shapes, gemm == M gemvs.
@@ -150,6 +155,28 @@ void nho_dequantize_row_q8_0(const void* vx, float* y, int64_t k) {
 			y[b * NHO_QK + j] = (float)qs[j] * d;
 		}
 	}
+}
+
+/* Token-embedding lookup: row ids[t] of the [n_rows x k] block matrix, dequantized, for every token
+ * (cpu/avx_2.hpp:80-103 prompt phase, :112-135 eval phase; per-op form :1241-1294).  The reference reads any row an
+ * id names; the GPU library defines an id outside [0, n_rows) as a row of zeros, restated here so both can be
+ * compared on such inputs.  Returns the number of such ids. */
+int64_t nho_get_rows_q8_0(const void* vw, const int32_t* ids, float* out, int64_t n_tokens, int64_t n_rows, int64_t k) {
+	const uint8_t* w	   = (const uint8_t*)vw;
+	const int64_t row_size = (k / NHO_QK) * NHO_BLOCK_BYTES;
+	int64_t invalid		   = 0;
+	for (int64_t t = 0; t < n_tokens; ++t) {
+		const int64_t id = ids[t];
+		if (id < 0 || id >= n_rows) {
+			for (int64_t j = 0; j < k; ++j) {
+				out[t * k + j] = 0.0f;
+			}
+			++invalid;
+			continue;
+		}
+		nho_dequantize_row_q8_0(w + id * row_size, out + t * k, k);
+	}
+	return invalid;
 }
 
 /* ---------------------------------------------------------------- quantize */

@@ -14,6 +14,7 @@ void nho_fill_activations(uint64_t seed, float* x, int64_t count);
 void nho_fill_weight_blocks(uint64_t seed, void* out, int64_t first_block, int64_t n_blocks);
 void nho_quantize_rows_q8_0(const float* x, void* y, int64_t m, int64_t k);
 void nho_gemm_q8_0(const void* w, const void* aq, float* c, int64_t m, int64_t n, int64_t k);
+int64_t nho_get_rows_q8_0(const void* w, const int32_t* ids, float* out, int64_t n_tokens, int64_t n_rows, int64_t k);
 }
 
 using namespace nihilus;
@@ -38,6 +39,13 @@ static_assert(k_mul_mat_op::input_01_dims[0] == K && k_mul_mat_op::output_dims[0
 static_assert(arch_index<device_types::gpu> == 5);
 static_assert(runtime_dims_t<k_mul_mat_op>);
 static_assert(sizeof(block_q8_0<half>) == NH_Q8_0_BLOCK_BYTES && Q_SIZE == NH_Q8_0_QK);
+
+// token embeddings: table [K, N rows] (the k-projection bytes stand in for an embedding table), ids [tokens], out [K, tokens]
+using ids_type		= core_trait_dims<test_config::max_sequence_length, 1, 1, 1>;
+using embd_out_dims = core_trait_dims<K, test_config::max_sequence_length, 1, 1, 1>;
+struct get_rows_op : kernel_traits_old<test_config, embd_out_dims, kernel_types::get_rows, float, weight_type, ids_type>, data_mixin<data_strategy_types::global, 32> {};
+using embd_eval_dispatch   = get_rows_dispatcher<test_config, processing_phases::eval_time, get_rows_op>;
+using embd_prompt_dispatch = get_rows_dispatcher<test_config, processing_phases::prompt_eval_time, get_rows_op>;
 
 using eval_dispatch	  = mul_mat_dispatcher<test_config, processing_phases::eval_time, k_mul_mat_op>;
 using prompt_dispatch = mul_mat_dispatcher<test_config, processing_phases::prompt_eval_time, k_mul_mat_op>;
@@ -122,6 +130,31 @@ int main(int argc, char** argv) {
 		thrown = std::strstr(e.what(), "null pointer") != nullptr;
 	}
 	REQUIRE(thrown);
+
+	// token embeddings: bit-exact, both phases, both table layouts; eval_time must honour the id
+	{
+		const int64_t T = 5;
+		const int32_t ids[T] = { 1023, 0, 17, 17, 512 };
+		std::vector<float> want_rows(T * K), got_rows(T * K);
+		REQUIRE(nho_get_rows_q8_0(w.data(), ids, want_rows.data(), T, N, K) == 0);
+		void *d_ids = nullptr, *d_e = nullptr;
+		REQUIRE(nh_malloc(&d_ids, sizeof(ids)) == NH_OK && nh_malloc(&d_e, test_config::max_sequence_length * K * 4) == NH_OK);
+		REQUIRE(nh_memcpy_h2d(d_ids, ids, sizeof(ids), nullptr) == NH_OK && nh_stream_sync(nullptr) == NH_OK);
+		get_rows_op e;
+		e.set_data(d_e);
+		e.get_seq_length_dim() = T;
+		for (const bool tiled : { false, true }) {
+			embd_prompt_dispatch::impl(e, tiled ? d_tiled : d_blocks, tiled, static_cast<const int32_t*>(d_ids));
+			REQUIRE(nh_memcpy_d2h(got_rows.data(), d_e, T * K * 4, nullptr) == NH_OK && nh_stream_sync(nullptr) == NH_OK);
+			REQUIRE(std::memcmp(got_rows.data(), want_rows.data(), T * K * 4) == 0);
+			embd_eval_dispatch::impl(e, tiled ? d_tiled : d_blocks, tiled, static_cast<const int32_t*>(d_ids) + 4); // id 512, not row 0
+			REQUIRE(nh_memcpy_d2h(got_rows.data(), d_e, K * 4, nullptr) == NH_OK && nh_stream_sync(nullptr) == NH_OK);
+			REQUIRE(std::memcmp(got_rows.data(), want_rows.data() + 4 * K, K * 4) == 0);
+		}
+		std::printf("get_rows         bit-exact (prompt and eval, blocks and tiled)\n");
+		nh_free(d_ids);
+		nh_free(d_e);
+	}
 
 	nh_free(d_blocks);
 	nh_free(d_tiled);
