@@ -78,6 +78,14 @@ int nh_q8_0_quantize(const float* x, void* xq_blocks, int64_t M, int64_t K, void
 /* Same values written in the tiled layout (rows padded with zero blocks to a multiple of 32). K % 128 == 0. */
 int nh_q8_0_quantize_tiled(const float* x, void* xq_tiled, int64_t M, int64_t K, void* stream);
 
+/* FFN activation fused into the quantizer: xq = quantize_row_q8_0(silu(gate) * up), element-wise over [M][K],
+ * silu(g) = g / (1 + exp(-g)).  Stands for the reference's ffn_silu -> ffn_gate_par (mul) -> activation operand of
+ * ffn_down chain (infra/core_traits.hpp:982-989; the silu and mul kernels are empty in the reference,
+ * cpu/avx_2.hpp:1946-2075, so the formula is the model's).  exp is evaluated as a fixed sequence of fp32 operations
+ * (see the CPU checker's nho_expf for the same sequence), which makes the quantized bytes reproducible bit for bit. */
+int nh_q8_0_silu_mul_quantize(const float* gate, const float* up, void* xq_blocks, int64_t M, int64_t K, void* stream);
+int nh_q8_0_silu_mul_quantize_tiled(const float* gate, const float* up, void* xq_tiled, int64_t M, int64_t K, void* stream);
+
 /* Layout conversion ---------------------------------------------------------------------------- */
 
 /* Bytes of a [rows x K] matrix: blocks = rows*(K/32)*34 (type_traits<block_q8_0>::total_byte_size,

@@ -25,6 +25,8 @@ SIGNATURES = {
     "nh_stream_sync": (_int, [_vp]),
     "nh_q8_0_quantize": (_int, [_vp, _vp, _i64, _i64, _vp]),
     "nh_q8_0_quantize_tiled": (_int, [_vp, _vp, _i64, _i64, _vp]),
+    "nh_q8_0_silu_mul_quantize": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
+    "nh_q8_0_silu_mul_quantize_tiled": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "nh_q8_0_blocks_bytes": (_i64, [_i64, _i64]),
     "nh_q8_0_tiled_bytes": (_i64, [_i64, _i64]),
     "nh_q8_0_tile": (_int, [_vp, _vp, _i64, _i64, _vp]),

@@ -214,6 +214,25 @@ int nh_q8_0_quantize_tiled(const float* x, void* xq_tiled, int64_t M, int64_t K,
 	return from_hip(nh::launch_quantize(x, xq_tiled, M, K, true, as_stream(stream)));
 }
 
+static int silu_mul_quantize_common(const float* gate, const float* up, void* xq, int64_t M, int64_t K, bool tiled, void* stream) {
+	NH_TRY(check_shape(M, 0, K, tiled));
+	if (M == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(gate && up && xq, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(gate) && aligned16(up) && aligned16(xq), NH_ERR_ALIGNMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_silu_mul_quantize(gate, up, xq, M, K, tiled, as_stream(stream)));
+}
+
+int nh_q8_0_silu_mul_quantize(const float* gate, const float* up, void* xq_blocks, int64_t M, int64_t K, void* stream) {
+	return silu_mul_quantize_common(gate, up, xq_blocks, M, K, false, stream);
+}
+
+int nh_q8_0_silu_mul_quantize_tiled(const float* gate, const float* up, void* xq_tiled, int64_t M, int64_t K, void* stream) {
+	return silu_mul_quantize_common(gate, up, xq_tiled, M, K, true, stream);
+}
+
 int nh_q8_0_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, void* stream) {
 	NH_TRY(check_shape(rows, 0, K, true));
 	if (rows == 0 || K == 0) {

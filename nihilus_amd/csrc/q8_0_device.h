@@ -73,6 +73,36 @@ __device__ __forceinline__ uint32_t quantize_block_lane(float4 v, uint16_t* dh) 
 	return q8(v.x) | (q8(v.y) << 8) | (q8(v.z) << 16) | (q8(v.w) << 24);
 }
 
+// exp(x) in fp32 as a fixed sequence of correctly rounded fp32 operations (multiply, fma, round-to-nearest-even,
+// exponent insertion), so that a host restatement of the same sequence gives the same bits: the activation that
+// feeds a quantizer must not depend on which math library evaluated it.  Range reduction by n = rne(x * log2 e) with
+// a two-part ln 2, degree-5 polynomial (the classic Cephes single-precision coefficients) on |r| <= ln2 / 2; within
+// 2 ulp of the true value.  The argument is clamped to [-87, 88] so that 2^n is a normal number.
+__device__ __forceinline__ float exp_f32(float x) {
+	x			  = fminf(fmaxf(x, -87.0f), 88.0f);
+	const float n = rintf(__fmul_rn(x, 1.44269504088896341f));
+	float r		  = fmaf(n, -0.693359375f, x);
+	r			  = fmaf(n, 2.12194440e-4f, r);
+	float p		  = 1.9875691500e-4f;
+	p			  = fmaf(p, r, 1.3981999507e-3f);
+	p			  = fmaf(p, r, 8.3334519073e-3f);
+	p			  = fmaf(p, r, 4.1665795894e-2f);
+	p			  = fmaf(p, r, 1.6666665459e-1f);
+	p			  = fmaf(p, r, 5.0000001201e-1f);
+	const float e = __fadd_rn(fmaf(p, __fmul_rn(r, r), r), 1.0f);
+	return __fmul_rn(e, __uint_as_float(static_cast<uint32_t>(static_cast<int>(n) + 127) << 23));
+}
+
+// SiLU(g) * u, the activation in front of the FFN down projection (ffn_silu -> ffn_gate_par in the reference's graph,
+// infra/core_traits.hpp:982-986; the reference's silu and mul kernels have no body, the formula is the model's:
+// silu(g) = g / (1 + exp(-g))).  IEEE divide, separate multiply.
+__device__ __forceinline__ float silu_mul(float g, float u) {
+	return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, exp_f32(-g))), u);
+}
+__device__ __forceinline__ float4 silu_mul4(float4 g, float4 u) {
+	return make_float4(silu_mul(g.x, u.x), silu_mul(g.y, u.y), silu_mul(g.z, u.z), silu_mul(g.w, u.w));
+}
+
 // Byte offset of macro-tile (strip, group) in a tiled matrix with `groups` = K/128 groups per strip.
 __device__ __host__ __forceinline__ int64_t macro_offset(int64_t strip, int64_t group, int64_t groups) {
 	return (strip * groups + group) * MACRO_BYTES;
@@ -101,6 +131,7 @@ inline hipError_t launch_kernel(int kind, Kernel kernel, dim3 grid, dim3 block, 
 // ---- launch functions (defined one per .hip file, called from q8_0_abi.hip after argument checks) ----
 
 hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s);
+hipError_t launch_silu_mul_quantize(const float* gate, const float* up, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s);
 hipError_t launch_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, hipStream_t s);
 hipError_t launch_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, hipStream_t s);
 hipError_t launch_get_rows(const void* W, const int32_t* ids, float* out, int32_t* invalid, int64_t n_tokens, int64_t n_rows, int64_t K, bool tiled, hipStream_t s);

@@ -13,7 +13,11 @@
 
 namespace nh {
 
-template<bool TILED> __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, uint8_t* __restrict__ out, int64_t M, int64_t rows_out, int64_t K) {
+//
+// SILU_MUL: the value quantized is silu(x) * u (the FFN activation in front of the down projection, computed from the
+// gate and up projections' outputs), so the fp32 activation never makes a round trip through memory.
+template<bool TILED, bool SILU_MUL>
+__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, const float* __restrict__ u, uint8_t* __restrict__ out, int64_t M, int64_t rows_out, int64_t K) {
 	const int64_t nb	= K / QK;
 	const int64_t t		= static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
 	const int64_t blk	= t >> 3; // block index over rows_out * nb
@@ -25,6 +29,9 @@ template<bool TILED> __global__ __launch_bounds__(256) void quantize_kernel(cons
 	float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 	if (in_range && m < M) {
 		v = *reinterpret_cast<const float4*>(x + m * K + b * QK + 4 * j);
+		if constexpr (SILU_MUL) {
+			v = silu_mul4(v, *reinterpret_cast<const float4*>(u + m * K + b * QK + 4 * j));
+		}
 	}
 	uint16_t dh;
 	const uint32_t packed = quantize_block_lane(v, &dh);
@@ -54,7 +61,7 @@ template<bool TILED> __global__ __launch_bounds__(256) void quantize_kernel(cons
 	}
 }
 
-hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s) {
+template<bool SILU_MUL> static hipError_t launch_quantize_t(const float* x, const float* u, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s) {
 	const int64_t rows_out = tiled ? (M + STRIP_ROWS - 1) / STRIP_ROWS * STRIP_ROWS : M;
 	const int64_t threads  = rows_out * (K / QK) * 8;
 	if (threads == 0) {
@@ -63,9 +70,17 @@ hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool
 	const int64_t grid = (threads + 255) / 256;
 	const dim3 g(static_cast<unsigned>(grid)), b(256);
 	if (tiled) {
-		return launch_kernel(KIND_QUANTIZE, quantize_kernel<true>, g, b, 0, s, x, static_cast<uint8_t*>(out), M, rows_out, K);
+		return launch_kernel(KIND_QUANTIZE, quantize_kernel<true, SILU_MUL>, g, b, 0, s, x, u, static_cast<uint8_t*>(out), M, rows_out, K);
 	}
-	return launch_kernel(KIND_QUANTIZE, quantize_kernel<false>, g, b, 0, s, x, static_cast<uint8_t*>(out), M, rows_out, K);
+	return launch_kernel(KIND_QUANTIZE, quantize_kernel<false, SILU_MUL>, g, b, 0, s, x, u, static_cast<uint8_t*>(out), M, rows_out, K);
+}
+
+hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s) {
+	return launch_quantize_t<false>(x, nullptr, out, M, K, tiled, s);
+}
+
+hipError_t launch_silu_mul_quantize(const float* gate, const float* up, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s) {
+	return launch_quantize_t<true>(gate, up, out, M, K, tiled, s);
 }
 
 } // namespace nh

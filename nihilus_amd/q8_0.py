@@ -52,6 +52,22 @@ def quantize_row_q8_0(x: torch.Tensor, tiled: bool = False) -> torch.Tensor:
     return out
 
 
+def silu_mul_quantize(gate: torch.Tensor, up: torch.Tensor, tiled: bool = False) -> torch.Tensor:
+    """quantize_row_q8_0(silu(gate) * up) for fp32 [M, K] (or [K]) operands, one kernel; output as quantize_row_q8_0."""
+    gate, up = _dev(gate, torch.float32, "gate"), _dev(up, torch.float32, "up")
+    if gate.shape != up.shape:
+        raise ValueError("gate and up must have the same shape")
+    g2 = gate.reshape(1, -1) if gate.dim() == 1 else gate
+    m, k = g2.shape
+    if tiled:
+        out = torch.empty(tiled_bytes(m, k), dtype=torch.uint8, device=gate.device)
+        _lib.check("nh_q8_0_silu_mul_quantize_tiled", _lib.lib().nh_q8_0_silu_mul_quantize_tiled(gate.data_ptr(), up.data_ptr(), out.data_ptr(), m, k, _stream()))
+        return out
+    out = torch.empty((m, blocks_bytes(1, k)), dtype=torch.uint8, device=gate.device)
+    _lib.check("nh_q8_0_silu_mul_quantize", _lib.lib().nh_q8_0_silu_mul_quantize(gate.data_ptr(), up.data_ptr(), out.data_ptr(), m, k, _stream()))
+    return out
+
+
 def tile(blocks: torch.Tensor, rows: int, k: int) -> torch.Tensor:
     blocks = _dev(blocks, torch.uint8, "blocks")
     if blocks.numel() != blocks_bytes(rows, k):

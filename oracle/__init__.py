@@ -52,6 +52,9 @@ _a_fp32_to_fp16 = _sig(_a, "nha_fp32_to_fp16", C.c_uint16, C.c_float)
 _q8_bytes = _sig(_o, "nho_q8_0_bytes", _i64, _i64, _i64)
 _dequant = _sig(_o, "nho_dequantize_row_q8_0", None, _vp, _vp, _i64)
 _get_rows = _sig(_o, "nho_get_rows_q8_0", _i64, _vp, _vp, _vp, _i64, _i64, _i64)
+_expf = _sig(_o, "nho_expf", C.c_float, C.c_float)
+_silu_mul = _sig(_o, "nho_silu_mul", C.c_float, C.c_float, C.c_float)
+_silu_mul_quant_rows = _sig(_o, "nho_silu_mul_quantize_rows_q8_0", None, _vp, _vp, _vp, _i64, _i64)
 _quant_rows = _sig(_o, "nho_quantize_rows_q8_0", None, _vp, _vp, _i64, _i64)
 _a_quant_rows = _sig(_a, "nha_quantize_rows_q8_0", None, _vp, _vp, _i64, _i64)
 _sums_gemv = _sig(_o, "nho_block_sums_gemv", None, _vp, _vp, _vp, _i64, _i64)
@@ -141,6 +144,28 @@ def get_rows(blocks: np.ndarray, ids: np.ndarray, n_rows: int, k: int):
     out = np.empty((ids.size, k), dtype=np.float32)
     bad = _get_rows(_ptr(b), _ptr(ids), _ptr(out), ids.size, n_rows, k)
     return out, int(bad)
+
+
+def expf(x: np.ndarray) -> np.ndarray:
+    """The checker's fixed-sequence fp32 exp, element-wise."""
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    return np.array([_expf(float(v)) for v in x], dtype=np.float32)
+
+
+def silu_mul(g: np.ndarray, u: np.ndarray) -> np.ndarray:
+    g = np.ascontiguousarray(g, dtype=np.float32).ravel()
+    u = np.ascontiguousarray(u, dtype=np.float32).ravel()
+    return np.array([_silu_mul(float(a), float(b)) for a, b in zip(g, u)], dtype=np.float32)
+
+
+def silu_mul_quantize_rows(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """gate, up: fp32 [m, k]; returns uint8 [m, (k//32)*34] = quantize_rows(silu(gate) * up)."""
+    g = np.ascontiguousarray(np.atleast_2d(gate), dtype=np.float32)
+    u = np.ascontiguousarray(np.atleast_2d(up), dtype=np.float32)
+    m, k = g.shape
+    out = np.empty((m, k // QK * BLOCK_BYTES), dtype=np.uint8)
+    _silu_mul_quant_rows(_ptr(g), _ptr(u), _ptr(out), m, k)
+    return out
 
 
 # ---------------------------------------------------------------- quantize

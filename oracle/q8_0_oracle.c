@@ -27,6 +27,9 @@
  *                                        decodes to the constant r (index order), out-of-range ids.  The
  *                                        reference's dump of this op's output (inp_embd) covers a vocabulary row
  *                                        whose bytes are not in the dumps, so it cannot be replayed end to end.
+ *   nho_expf / nho_silu_mul              no reference body exists (its silu kernels are empty): pinned against the
+ *                                        correctly rounded double-precision value, <= 2 ulp over a dense sweep of
+ *                                        the whole clamped range plus the special points; silu against float64.
  *   nho_block_sum_i32                    int64 brute force; extreme blocks (+-127 -> +-516128).
  *   nho_vec_dot_* / gemv / gemm          float64 evaluation (<= ~1e-6 rel), d == 1 gives exact
  *                                        integers, tiny hand-checkable shapes, gemm == M gemvs.
@@ -177,6 +180,61 @@ int64_t nho_get_rows_q8_0(const void* vw, const int32_t* ids, float* out, int64_
 		nho_dequantize_row_q8_0(w + id * row_size, out + t * k, k);
 	}
 	return invalid;
+}
+
+/* ---------------------------------------------------------------- FFN activation */
+
+void nho_quantize_row_q8_0(const float* x, void* vy, int64_t k);
+
+/* exp(x) as a fixed sequence of correctly rounded fp32 operations: n = rne(x * log2 e), two-part ln 2 reduction by
+ * fma, degree-5 polynomial (Cephes single-precision coefficients) by fma, 2^n by exponent insertion; argument clamped
+ * to [-87, 88].  Not a restatement of reference code (the reference's silu kernels are empty, cpu/avx_2.hpp:1946-2075):
+ * it exists so that the GPU and this checker evaluate the model's SiLU with the same bits.  Pinned against the
+ * correctly rounded value (double exp) to <= 2 ulp over a dense sweep. */
+float nho_expf(float x) {
+	x				 = fminf(fmaxf(x, -87.0f), 88.0f);
+	volatile float t = x * 1.44269504088896341f;
+	const float n	 = nearbyintf(t);
+	float r			 = fmaf(n, -0.693359375f, x);
+	r				 = fmaf(n, 2.12194440e-4f, r);
+	float p			 = 1.9875691500e-4f;
+	p				 = fmaf(p, r, 1.3981999507e-3f);
+	p				 = fmaf(p, r, 8.3334519073e-3f);
+	p				 = fmaf(p, r, 4.1665795894e-2f);
+	p				 = fmaf(p, r, 1.6666665459e-1f);
+	p				 = fmaf(p, r, 5.0000001201e-1f);
+	volatile float r2 = r * r;
+	volatile float e  = fmaf(p, r2, r);
+	e				  = e + 1.0f;
+	union {
+		uint32_t u;
+		float f;
+	} two_n;
+	two_n.u = (uint32_t)((int32_t)n + 127) << 23;
+	return e * two_n.f;
+}
+
+/* silu(g) * u with silu(g) = g / (1 + exp(-g)): ffn_silu then ffn_gate_par (mul) of the reference's graph
+ * (infra/core_traits.hpp:982-986); IEEE divide, separate multiply. */
+float nho_silu_mul(float g, float u) {
+	volatile float den = 1.0f + nho_expf(-g);
+	volatile float s   = g / den;
+	return s * u;
+}
+
+/* xq = quantize_row_q8_0(silu(gate) * up), m rows of k */
+void nho_silu_mul_quantize_rows_q8_0(const float* gate, const float* up, void* vy, int64_t m, int64_t k) {
+	float act[NHO_QK];
+	uint8_t* y		 = (uint8_t*)vy;
+	const int64_t nb = k / NHO_QK;
+	for (int64_t r = 0; r < m; ++r) {
+		for (int64_t b = 0; b < nb; ++b) {
+			for (int j = 0; j < NHO_QK; ++j) {
+				act[j] = nho_silu_mul(gate[r * k + b * NHO_QK + j], up[r * k + b * NHO_QK + j]);
+			}
+			nho_quantize_row_q8_0(act, y + (r * nb + b) * NHO_BLOCK_BYTES, NHO_QK);
+		}
+	}
 }
 
 /* ---------------------------------------------------------------- quantize */
