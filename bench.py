@@ -31,7 +31,8 @@ GATE_N, HIDDEN, FFN = 14336, 4096, 14336
 # HBM bytes per launch of the dominant kernel, mean over the step's two launches: FETCH_SIZE and WRITE_SIZE from two
 # rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for a plain 64 MiB copy
 # (FETCH_SIZE x 1.99928, WRITE_SIZE x 1.0).  A hardware-counter figure cannot be taken live; this is the recorded one.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 93907580
+# Keyed by --ffn-mode; None = not measured yet for that mode.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"batch": 93907580, "fused": None}
 
 
 def weight_bytes(n: int, k: int) -> int:
@@ -63,6 +64,10 @@ def main() -> int:
     ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
+    ap.add_argument("--ffn-mode", choices=["batch", "fused"], default="batch",
+                    help="batch (default): the step's three mat-vecs through nh_q8_0_mul_mat_batch as two launches, the down projection fed from a "
+                    "resident fp32 vector (mat-vecs only, as the metric is defined).  fused: the step as one launch (nh_q8_0_ffn_f32: gate, up, "
+                    "SiLU*up, down), which the default run reports beside the headline as `ffn_one_launch`")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode-step leg (8 GB of weights)")
     ap.add_argument("--decode-tokens", type=int, default=200, help="timed tokens of the decode-step leg")
     ap.add_argument("--roofline-steps", type=int, default=0, help="steps of the per-kernel timing pass (default: min(steps, 1000))")
@@ -129,14 +134,28 @@ def main() -> int:
     batch = lib.nh_q8_0_mul_mat_batch
     ws_ptr, ws_n = ws.data_ptr(), ws.numel()
 
+    fused = args.ffn_mode == "fused"
+    ffn = lib.nh_q8_0_ffn_f32
+    ptrs = [(m[0].data_ptr(), m[1].data_ptr(), m[2].data_ptr()) for m in layers]
+    x_ptr, y_ptr = x.data_ptr(), y_down.data_ptr()
+
     def run_steps(count: int, start: int = 0) -> None:
         for i in range(start, start + count):
-            rc = batch(op_lists[i % L], 3, ws_ptr, ws_n, stream)
+            if fused:
+                g, u, d = ptrs[i % L]
+                rc = ffn(g, u, d, x_ptr, None, y_ptr, FFN, HIDDEN, HIDDEN, stream)
+            else:
+                rc = batch(op_lists[i % L], 3, ws_ptr, ws_n, stream)
             if rc != 0:
-                _lib.check("nh_q8_0_mul_mat_batch", rc)
+                _lib.check("nh_q8_0_ffn_f32" if fused else "nh_q8_0_mul_mat_batch", rc)
 
-    # the batch runner turns the step into two launches: gate+up (shared x) and down, each with its quantize inside
-    launch_bytes_list = [fused_launch_bytes([GATE_N, GATE_N], HIDDEN), fused_launch_bytes([HIDDEN], FFN)]
+    # algorithmic bytes of the step: every weight block once, the fp32 activation rows read, the fp32 outputs written.
+    # batch mode: two launches, gate+up (shared x) and down, each with its quantize inside.  fused mode: one launch; the
+    # gate/up outputs (2 x 57 KB) stay inside the launch and are not counted.
+    if fused:
+        launch_bytes_list = [fused_launch_bytes([GATE_N, GATE_N], HIDDEN) - 8 * GATE_N + fused_launch_bytes([HIDDEN], FFN) - 4 * FFN]
+    else:
+        launch_bytes_list = [fused_launch_bytes([GATE_N, GATE_N], HIDDEN), fused_launch_bytes([HIDDEN], FFN)]
     step_bytes = sum(launch_bytes_list)
 
     # ---------------------------------------------------------------- warm-up, then EXACTLY --steps timed steps
@@ -158,10 +177,10 @@ def main() -> int:
     launch_bytes = step_bytes / len(launch_bytes_list)  # mean over the step's launches of the dominant kernel
     avg_ms = tot.value / max(1, cnt.value)
     achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
-    assert cnt.value == len(launch_bytes_list) * rsteps, "the step is expected to be two mat-vec launches"
+    assert cnt.value == len(launch_bytes_list) * rsteps, "unexpected number of mat-vec launches per step"
 
     # sanity: the last step's outputs are finite (a wrong kernel would usually show up here first)
-    finite = bool(torch.isfinite(y_gate).all() and torch.isfinite(y_up).all() and torch.isfinite(y_down).all())
+    finite = bool(torch.isfinite(y_down).all() and (fused or (torch.isfinite(y_gate).all() and torch.isfinite(y_up).all())))
 
     result = {
         "metric": "Q8_0 GEMV HBM GB/s (% of peak) + LLaMA-3-8B-shape decode tok/s, 1 GPU",
@@ -177,7 +196,8 @@ def main() -> int:
         "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate",
         "data": "synthetic",
         "config": {
-            "workload": "LLaMA-3-8B FFN decode GEMVs, batch 1: gate+up Q8_0 [14336x4096], down Q8_0 [4096x14336], activation quantize included",
+            "workload": "LLaMA-3-8B FFN decode GEMVs, batch 1: gate+up Q8_0 [14336x4096], down Q8_0 [4096x14336], activation quantize included"
+            + (", SiLU(gate)*up feeding down, one launch per step" if fused else ", two launches per step"),
             "weight_sets_rotated": L,
             "bytes_per_step": step_bytes,
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
@@ -185,13 +205,14 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "nh::gemv_tiled_kernel<TILES, XF32=true> (streaming mat-vec with the activation quantize inside; "
-            "two launches per step: gate+up as one 125 MB launch, down as one 62 MB launch)",
+            "kernel": ("nh::ffn_decode_kernel<TILES=2> (gate, up and down mat-vecs of the step as one 187 MB launch, activation quantize and SiLU*up inside)"
+                       if fused else "nh::gemv_tiled_kernel<TILES, XF32=true> (streaming mat-vec with the activation quantize inside; "
+                       "two launches per step: gate+up as one 125 MB launch, down as one 62 MB launch)"),
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH[args.ffn_mode],
             "bytes_per_launch": launch_bytes,
             "avg_launch_us": round(avg_ms * 1e3, 3),
             "min_launch_us": round(mn.value * 1e3, 3),
@@ -199,6 +220,21 @@ def main() -> int:
             "launches_timed": cnt.value,
         },
     }
+
+    if not fused:
+        # the same step as ONE launch with the real dependency inside (down fed by silu(gate) * up): reported beside the headline
+        fb = fused_launch_bytes([GATE_N, GATE_N], HIDDEN) - 8 * GATE_N + fused_launch_bytes([HIDDEN], FFN) - 4 * FFN
+        fused = True
+        run_steps(args.warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(args.steps, start=args.warmup)
+        torch.cuda.synchronize()
+        f_sec = (time.perf_counter() - t0) / args.steps
+        result["ffn_one_launch"] = {"entry": "nh_q8_0_ffn_f32", "ms_per_step": round(f_sec * 1e3, 6), "GBs": round(fb / f_sec / 1e9, 1),
+                                    "pct_of_hbm_peak": round(100.0 * fb / f_sec / 1e9 / HBM_PEAK_GBS, 2), "bytes_per_step": fb,
+                                    "outputs_finite": bool(torch.isfinite(y_down).all())}
+        fused = False
 
     del layers, op_lists
     torch.cuda.empty_cache()

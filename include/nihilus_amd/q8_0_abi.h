@@ -126,6 +126,19 @@ int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_
  * as ONE launch: y[i] = W_tiled[i] . quantize(x), i < count.  host_* arrays are host memory, read before return. */
 int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream);
 
+/* The decode-time FFN as one launch:  y = W_down . Q(silu(W_gate . Q(x)) * (W_up . Q(x))) [+ residual],  Q = quantize_row_q8_0.
+ * Stands for the eval_time body of the reference's mega_ffn core: ffn_gate and ffn_up mul_mat, silu, mul, ffn_down
+ * mul_mat, residual add (infra/core_traits.hpp:971-995; the GPU dispatcher that would hold it is empty,
+ * cuda/cuda_12.hpp:806-916).  Same arithmetic, bit for bit, as nh_q8_0_gemv_tiled_multi_f32 (gate, up) followed by
+ * nh_q8_0_silu_mul_quantize and nh_q8_0_gemv_tiled (down): the down projection's workgroups ride in the same grid
+ * and start streaming their weights while gate/up are still running.
+ * W_gate, W_up: [N_ff x K] tiled; W_down: [N_out x N_ff] tiled; x: fp32 [K]; residual: fp32 [N_out] or NULL;
+ * y: fp32 [N_out] (may alias residual).  K % 128 == 0, N_ff % 128 == 0, N_ff <= NH_Q8_0_FFN_MAX_HIDDEN.
+ * Uses the library's per-device scratch: two such calls must not overlap on one GPU. */
+#define NH_Q8_0_FFN_MAX_HIDDEN 65536
+int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* residual, float* y, int64_t N_ff, int64_t K, int64_t N_out,
+	void* stream);
+
 /* Mat-mat (prefill, prompt_eval_time) ----------------------------------------------------------- */
 
 /* C[m*N + n] (n fastest, ggml's dst[ir1*nr0 + ir0], cpu/avx_2.hpp:4934) = the same dot for activation
@@ -181,6 +194,9 @@ int nh_q8_0_debug_block_sums(const void* W, const void* Aq, int32_t* sums, int64
 
 /* What the fused mat-vec stages for x: runs the fused kernel's own quantize-and-stage code on fp32 x [K] and writes
  * the staged row back as K/32 packed blocks, to be compared byte for byte with nh_q8_0_quantize. K % 128 == 0. */
+/* The gate and up projections' fp32 outputs of the last nh_q8_0_ffn_f32 on this device (they never leave the
+ * library otherwise), copied out for comparison. */
+int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void* stream);
 int nh_q8_0_debug_fused_quantize(const float* x, void* xq_blocks_out, int64_t K, void* stream);
 
 /* Synthetic inputs (benchmark / test utility) --------------------------------------------------- */

@@ -276,6 +276,35 @@ int nh_q8_0_get_rows_tiled(const void* W_tiled, const int32_t* ids, float* out, 
 	return get_rows_common(W_tiled, ids, out, invalid_count, n_tokens, n_rows, K, true, stream);
 }
 
+int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* residual, float* y, int64_t N_ff, int64_t K, int64_t N_out,
+	void* stream) {
+	NH_TRY(check_shape(N_ff, 0, K, true)); // gate, up: [N_ff x K]
+	NH_TRY(check_shape(N_out, 0, N_ff, true)); // down: [N_out x N_ff]
+	NH_REQUIRE(N_ff <= NH_Q8_0_FFN_MAX_HIDDEN, NH_ERR_TOO_LARGE);
+	if (N_out == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(y, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
+	if (N_ff > 0 && K > 0) {
+		NH_REQUIRE(W_gate_tiled && W_up_tiled && W_down_tiled && x, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(W_gate_tiled) && aligned16(W_up_tiled) && aligned16(W_down_tiled) && aligned16(x), NH_ERR_ALIGNMENT);
+	}
+	NH_TRY(require_device());
+	return from_hip(nh::launch_ffn_decode(W_gate_tiled, W_up_tiled, W_down_tiled, x, residual, y, N_ff, K, N_out, as_stream(stream)));
+}
+
+int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void* stream) {
+	NH_REQUIRE(N_ff >= 0, NH_ERR_SHAPE);
+	NH_REQUIRE(N_ff <= NH_Q8_0_FFN_MAX_HIDDEN, NH_ERR_TOO_LARGE);
+	if (N_ff == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(gate_out && up_out, NH_ERR_NULL_POINTER);
+	NH_TRY(require_device());
+	return from_hip(nh::copy_ffn_gate_up(gate_out, up_out, N_ff, as_stream(stream)));
+}
+
 static int gemv_common(const void* W, const void* xq, float* y, int64_t N, int64_t K, bool tiled, void* stream) {
 	NH_TRY(check_shape(N, 0, K, tiled));
 	NH_REQUIRE(tiled || K <= MAX_K_BLOCKS_GEMV, NH_ERR_TOO_LARGE);

@@ -103,6 +103,14 @@ __device__ __forceinline__ float4 silu_mul4(float4 g, float4 u) {
 	return make_float4(silu_mul(g.x, u.x), silu_mul(g.y, u.y), silu_mul(g.z, u.z), silu_mul(g.w, u.w));
 }
 
+// Blocks the wave until every memory operation it has issued, stores included, has been acknowledged.  Placed
+// between device-scope (write-through) stores of data and the device-scope store or atomic that tells another
+// workgroup the data is there: a workgroup-scope release fence does not wait for the stores on this target, and an
+// agent-scope one also writes back the L2 under the other workgroups' streaming loads.
+__device__ __forceinline__ void wait_stores_acknowledged() {
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // Byte offset of macro-tile (strip, group) in a tiled matrix with `groups` = K/128 groups per strip.
 __device__ __host__ __forceinline__ int64_t macro_offset(int64_t strip, int64_t group, int64_t groups) {
 	return (strip * groups + group) * MACRO_BYTES;
@@ -145,6 +153,9 @@ hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* 
 constexpr int GEMV_MAX_SEGMENTS = 3;
 hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s);
 // Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
+hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* residual, float* y, int64_t n_ff, int64_t K, int64_t n_out,
+	hipStream_t s);
+hipError_t copy_ffn_gate_up(float* gate_out, float* up_out, int64_t n_ff, hipStream_t s);
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s);
 hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s);
 // Tiled operands, M <= GEMM_SKINNY_MAX_M: the HBM-streaming MFMA kernel for batched decode (q8_0_gemm_skinny.hip).

@@ -1,0 +1,279 @@
+// The decode-time FFN as ONE launch: y = W_down . Q(silu(W_gate . Q(x)) * (W_up . Q(x))) [+ residual], gfx950.
+//
+// Stands for the eval_time body of the reference's mega_ffn core (ffn_gate/ffn_up mul_mat -> silu -> mul -> ffn_down
+// mul_mat -> residual add, infra/core_traits.hpp:971-995; its GPU dispatcher is empty, cuda/cuda_12.hpp:806-916).
+// Every Q() is quantize_row_q8_0 done inside the consuming mat-vec, so no activation is ever written in quantized form.
+//
+// Why one launch: the three mat-vecs are HBM-bound and each launch pays a ramp (first bytes ~2 us after the launch
+// starts) and a tail (the last workgroups run on a mostly idle chip).  Here the workgroups of the down projection are
+// part of the same grid, placed after those of gate and up.  A down-projection wave puts all its weight loads in flight
+// the moment it starts -- while gate/up workgroups are still streaming -- and only then waits for the activation
+// blocks that cover its slice, so HBM never idles between the two phases.
+//
+// A producer workgroup computes the SAME 32-row strip of gate (waves 0-7) and of up (waves 8-15): those 32 + 32 outputs
+// are exactly what one 32-value block of the down projection's activation needs, so the producer applies silu(g) * u,
+// quantizes the block (the quantize kernel's arithmetic) and publishes 34 bytes; consumers never evaluate an exp and
+// read 1/7.5 of what the fp32 vectors would cost them.
+//
+// Progress: workgroups are dispatched in index order within each XCD's share of the grid, and producers all precede
+// consumers, so a waiting consumer never keeps a producer from being scheduled; producers wait for nothing.  The wait
+// is bounded all the same (see gemv_chunk).  Hand-off: a producer publishes its block with device-scope stores, waits
+// for the acknowledgements, then stores the launch's epoch into the block's flag; nothing is reset between launches
+// (epochs only move forward).
+#include "q8_0_gemv_tiled.h"
+
+namespace nh {
+
+struct ffn_args {
+	const uint8_t* w_gate;
+	const uint8_t* w_up;
+	const uint8_t* w_down;
+	const float* x; // [K]
+	const float* residual; // [n_out] or null
+	float* y; // [n_out]
+	float* gate_up; // scratch: g at [0, n_ff), u at [FFN_MAX_HIDDEN, FFN_MAX_HIDDEN + n_ff), kept for inspection
+	uint32_t* act_q; // scratch: the activation's quants, 8 dwords per block
+	float* act_d; // scratch: its scales
+	unsigned* flags; // scratch: one word per block
+	unsigned epoch;
+	float* partials;
+	unsigned* counters;
+	int n_ff, n_out;
+	int groups_p, groups_c; // K / 128, n_ff / 128
+	int producers; // n_ff / 32
+	int p_per_slot, p_rem; // a producer strip's K range over the 8 waves of one matrix
+	int split_shift, c_per_slot, c_rem; // a consumer strip's K range over splits * 16 waves
+};
+
+template<int TILES, bool LOOP> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
+	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K];
+	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
+	__shared__ float red[GEMV_WAVES][64];
+	__shared__ int last_flag;
+
+	const int tid  = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wg   = static_cast<int>(blockIdx.x);
+
+	if (wg < a.producers) {
+		// ---- rows [32 * wg, 32 * wg + 32) of gate (waves 0-7) and of up (waves 8-15) -> activation block wg ----
+		__shared__ __align__(16) float act_f[STRIP_ROWS];
+		const int matrix	   = wave >> 3;
+		const int slot		   = wave & 7;
+		const int strip		   = wg;
+		const int g0		   = slot * a.p_per_slot + min(slot, a.p_rem);
+		const int g1		   = g0 + a.p_per_slot + (slot < a.p_rem ? 1 : 0);
+		const uint8_t* w_strip = (matrix ? a.w_up : a.w_gate) + macro_offset(strip, 0, a.groups_p);
+		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
+		float acc			   = 0.0f;
+		if constexpr (!LOOP) {
+			acc = gemv_chunk<TILES, X_F32, DUMP_NONE>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false);
+		} else {
+			for (int gc = g0; gc < g1; gc += TILES) {
+				acc += gemv_chunk<TILES, X_F32, DUMP_NONE>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false);
+				__builtin_amdgcn_wave_barrier();
+			}
+		}
+		red[wave][lane] = acc;
+		__syncthreads();
+		if (wave == 0) {
+			if (lane < STRIP_ROWS) {
+				float g = 0.0f, u = 0.0f;
+#pragma unroll
+				for (int w = 0; w < GEMV_WAVES / 2; ++w) {
+					g += red[w][lane] + red[w][32 + lane];
+					u += red[GEMV_WAVES / 2 + w][lane] + red[GEMV_WAVES / 2 + w][32 + lane];
+				}
+				act_f[lane]									 = silu_mul(g, u);
+				a.gate_up[strip * STRIP_ROWS + lane]				 = g; // inspection copies, not read by this launch
+				a.gate_up[FFN_MAX_HIDDEN + strip * STRIP_ROWS + lane] = u;
+			}
+			__builtin_amdgcn_wave_barrier();
+			// the block as eight float4 in lanes 0..7; every lane runs the quantizer (lanes 8.. on zeros)
+			const float4 v = lane < 8 ? *reinterpret_cast<const float4*>(&act_f[4 * lane]) : make_float4(0.f, 0.f, 0.f, 0.f);
+			uint16_t dh;
+			const uint32_t packed = quantize_block_lane(v, &dh);
+			if (lane < 8) {
+				__hip_atomic_store(&a.act_q[strip * 8 + lane], packed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
+			if (lane == 0) {
+				__hip_atomic_store(&a.act_d[strip], half_bits_to_float(dh), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
+			wait_stores_acknowledged();
+			if (lane == 0) {
+				__hip_atomic_store(&a.flags[strip], a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
+		}
+		return;
+	}
+
+	// ---- a (32-row strip, K split) of the down projection; its activation blocks come from the producers ----
+	const int c		 = wg - a.producers;
+	const int splits = 1 << a.split_shift;
+	const int gstrip = c >> a.split_shift;
+	const int split	 = c & (splits - 1);
+	const int slot	 = split * GEMV_WAVES + wave;
+	const int g0	 = slot * a.c_per_slot + min(slot, a.c_rem);
+	const int g1	 = g0 + a.c_per_slot + (slot < a.c_rem ? 1 : 0);
+
+	const uint8_t* w_strip = a.w_down + macro_offset(gstrip, 0, a.groups_c);
+	const int row_l		   = gstrip * STRIP_ROWS + (lane & 31);
+	float acc			   = 0.0f;
+	if constexpr (!LOOP) {
+		acc = gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_q, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_c, lane, row_l, a.n_out, false, a.act_d, a.flags,
+			a.epoch);
+	} else {
+		for (int gc = g0; gc < g1; gc += TILES) {
+			acc += gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_q, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_c, lane, row_l, a.n_out, false,
+				a.act_d, a.flags, a.epoch);
+			__builtin_amdgcn_wave_barrier();
+		}
+	}
+
+	red[wave][lane] = acc;
+	__syncthreads();
+	float total = 0.0f;
+	if (tid < STRIP_ROWS) {
+#pragma unroll
+		for (int w = 0; w < GEMV_WAVES; ++w) {
+			total += red[w][tid] + red[w][32 + tid];
+		}
+	}
+	const int row = gstrip * STRIP_ROWS + tid;
+	if (splits == 1) {
+		if (tid < STRIP_ROWS && row < a.n_out) {
+			a.y[row] = a.residual ? total + a.residual[row] : total;
+		}
+		return;
+	}
+	// K split over several workgroups: as in the plain mat-vec, the last to arrive adds the partial sums in split order
+	if (tid < STRIP_ROWS) {
+		__hip_atomic_store(&a.partials[(static_cast<int64_t>(gstrip) * splits + split) * STRIP_ROWS + tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+	}
+	wait_stores_acknowledged();
+	__syncthreads();
+	if (tid == 0) {
+		const unsigned prev = __hip_atomic_fetch_add(&a.counters[gstrip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		const int last		= (prev == static_cast<unsigned>(splits - 1));
+		if (last) {
+			__hip_atomic_store(&a.counters[gstrip], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		}
+		last_flag = last;
+	}
+	__syncthreads();
+	if (last_flag && tid < STRIP_ROWS && row < a.n_out) {
+		const float* mine = a.partials + static_cast<int64_t>(gstrip) * splits * STRIP_ROWS + tid;
+		float sum		  = 0.0f;
+		for (int sp0 = 0; sp0 < splits; sp0 += 8) {
+			float v[8];
+#pragma unroll
+			for (int u = 0; u < 8; ++u) {
+				v[u] = (sp0 + u < splits) ? __hip_atomic_load(&mine[(sp0 + u) * STRIP_ROWS], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+			}
+#pragma unroll
+			for (int u = 0; u < 8; ++u) {
+				if (sp0 + u < splits) {
+					sum += v[u];
+				}
+			}
+		}
+		a.y[row] = a.residual ? sum + a.residual[row] : sum;
+	}
+}
+
+// an empty inner dimension anywhere makes the activation zero: y = residual (or 0)
+__global__ void ffn_empty_kernel(float* __restrict__ y, const float* __restrict__ residual, int64_t n) {
+	const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+	if (i < n) {
+		y[i] = residual ? residual[i] : 0.0f;
+	}
+}
+
+template<int TILES, bool LOOP> static hipError_t launch_ffn_t(const ffn_args& a, unsigned grid, hipStream_t s) {
+	return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
+}
+
+// n_ff % 128 == 0, K % 128 == 0, n_ff <= FFN_MAX_HIDDEN (checked by the caller).
+hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* residual, float* y, int64_t n_ff, int64_t K, int64_t n_out,
+	hipStream_t s) {
+	if (n_out == 0) {
+		return hipSuccess;
+	}
+	if (n_ff == 0 || K == 0) {
+		ffn_empty_kernel<<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, s>>>(y, residual, n_out);
+		return hipGetLastError();
+	}
+	gemv_scratch sc;
+	const hipError_t e = get_gemv_scratch(&sc, true);
+	if (e != hipSuccess) {
+		return e;
+	}
+	// the down projection: K over as many workgroups per strip as it takes for a wave to own at most 4 groups
+	const int strips_c = static_cast<int>((n_out + STRIP_ROWS - 1) / STRIP_ROWS);
+	const int groups_c = static_cast<int>(n_ff / GROUP_K);
+	int splits		   = 1;
+	auto tiles_for	   = [&](int sp) { return (groups_c + GEMV_WAVES * sp - 1) / (GEMV_WAVES * sp); };
+	while (tiles_for(splits) > 4 && strips_c <= GEMV_MAX_SPLIT_STRIPS && strips_c * splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
+		splits *= 2;
+	}
+	ffn_args a{};
+	a.w_gate	 = static_cast<const uint8_t*>(w_gate);
+	a.w_up		 = static_cast<const uint8_t*>(w_up);
+	a.w_down	 = static_cast<const uint8_t*>(w_down);
+	a.x			 = x;
+	a.residual	 = residual;
+	a.y			 = y;
+	a.gate_up	 = sc.gate_up;
+	a.act_q		 = sc.act_q;
+	a.act_d		 = sc.act_d;
+	a.flags		 = sc.flags;
+	a.epoch		 = sc.epoch;
+	a.partials	 = sc.partials;
+	a.counters	 = sc.counters;
+	a.n_ff		 = static_cast<int>(n_ff);
+	a.n_out		 = static_cast<int>(n_out);
+	a.groups_p	 = static_cast<int>(K / GROUP_K);
+	a.groups_c	 = groups_c;
+	a.producers	 = static_cast<int>(n_ff / STRIP_ROWS);
+	a.p_per_slot = a.groups_p / (GEMV_WAVES / 2);
+	a.p_rem		 = a.groups_p % (GEMV_WAVES / 2);
+	int shift	 = 0;
+	while ((1 << shift) < splits) {
+		++shift;
+	}
+	const int slots		= splits * GEMV_WAVES;
+	a.split_shift		= shift;
+	a.c_per_slot		= a.groups_c / slots;
+	a.c_rem				= a.groups_c % slots;
+	const int tiles_p	= (a.groups_p + GEMV_WAVES / 2 - 1) / (GEMV_WAVES / 2);
+	const int tiles_c	= tiles_for(splits);
+	const int tiles		= tiles_p > tiles_c ? tiles_p : tiles_c;
+	const unsigned grid = static_cast<unsigned>(a.producers + strips_c * splits);
+	if (tiles > 4) {
+		return launch_ffn_t<4, true>(a, grid, s);
+	}
+	if (tiles <= 1) {
+		return launch_ffn_t<1, false>(a, grid, s);
+	}
+	if (tiles <= 2) {
+		return launch_ffn_t<2, false>(a, grid, s);
+	}
+	return launch_ffn_t<4, false>(a, grid, s);
+}
+
+// parity hook: the gate and up projections' outputs of the last fused launch on this device
+hipError_t copy_ffn_gate_up(float* gate_out, float* up_out, int64_t n_ff, hipStream_t s) {
+	gemv_scratch sc;
+	hipError_t e = get_gemv_scratch(&sc);
+	if (e != hipSuccess) {
+		return e;
+	}
+	e = hipMemcpyAsync(gate_out, sc.gate_up, static_cast<size_t>(n_ff) * 4, hipMemcpyDeviceToDevice, s);
+	if (e != hipSuccess) {
+		return e;
+	}
+	return hipMemcpyAsync(up_out, sc.gate_up + FFN_MAX_HIDDEN, static_cast<size_t>(n_ff) * 4, hipMemcpyDeviceToDevice, s);
+}
+
+} // namespace nh

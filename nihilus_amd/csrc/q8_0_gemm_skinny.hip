@@ -171,7 +171,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 			}
 		}
 	}
-	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // the stores have completed (written through) before the arrival is counted
+	wait_stores_acknowledged();
 	__syncthreads();
 	if (tid == 0) {
 		const unsigned prev = __hip_atomic_fetch_add(&counters[strip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -11,7 +11,7 @@
 //   gemv_tiled_kernel   the streaming kernel on the tiled layout -- the one the decode path runs.
 // In both, lane l accumulates row (l % 32), quants 16*(l/32).. of every block, so the loop needs no cross-lane
 // reduction; halves and waves are combined once through LDS in a fixed order (run-to-run bit-stable).
-#include "q8_0_device.h"
+#include "q8_0_gemv_tiled.h"
 
 #include <mutex>
 
@@ -115,142 +115,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* 
 //     depend on arrival order;
 //   * up to three weight matrices that share K and the activation row (q/k/v, gate/up) run as one launch:
 //     a bigger launch amortises the ramp-up and the tail.
-constexpr int GEMV_WAVES = 16;
-
-struct gemv_segments {
-	const uint8_t* W[GEMV_MAX_SEGMENTS];
-	float* y[GEMV_MAX_SEGMENTS];
-	int rows[GEMV_MAX_SEGMENTS];
-	int strip_end[GEMV_MAX_SEGMENTS]; // running total of strips
-};
-
-enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
-
-// One chunk of a wave's K range: groups [gc, gc + cnt), cnt <= TILES, all wave-uniform (scalar registers).
-// xs_q / xs_d are this wave's private LDS slices.  Returns the lane's partial dot product over the chunk.
-template<int TILES, bool XF32, int DUMP>
-__device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
-	int groups, int lane, int row, int N, bool dump_this_strip) {
-	const int r	   = lane & 31;
-	const int half = lane >> 5;
-
-	// ---- 1. activation slice loads, issued first ----
-	constexpr int XQ_LOADS = (TILES * 34 + 63) / 64; // raw dwords of blocks [4*gc, 4*(gc+cnt)): 34 dwords per group
-	constexpr int XF_LOADS = (TILES * 32 + 63) / 64; // float4 per lane: 128 floats per group = 32 float4
-	uint32_t xr[XQ_LOADS];
-	float4 xf[XF_LOADS];
-	if constexpr (XF32) {
-		const float4* x4 = reinterpret_cast<const float4*>(static_cast<const float*>(xin) + static_cast<int64_t>(gc) * GROUP_K);
-#pragma unroll
-		for (int i = 0; i < XF_LOADS; ++i) {
-			const int v = lane + 64 * i; // float4 index in the slice; block = v / 8
-			xf[i]		= v < cnt * 32 ? x4[v] : make_float4(0.f, 0.f, 0.f, 0.f);
-		}
-	} else {
-		const uint32_t* x_raw = reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(xin) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * BLOCK_BYTES));
-#pragma unroll
-		for (int i = 0; i < XQ_LOADS; ++i) {
-			const int v = lane + 64 * i;
-			xr[i]		= v < cnt * 34 ? x_raw[v] : 0u;
-		}
-	}
-
-	// ---- 2. every weight byte of the chunk, in flight at once ----
-	v4i q[TILES][GROUP_BLOCKS];
-	v2u dd[TILES];
-	if constexpr (DUMP != DUMP_X) {
-		const uint8_t* macro0 = w_strip + static_cast<int64_t>(gc) * MACRO_BYTES;
-#pragma unroll
-		for (int t = 0; t < TILES; ++t) {
-			if (t < cnt) {
-				const uint8_t* macro = macro0 + t * MACRO_BYTES;
-#pragma unroll
-				for (int j = 0; j < GROUP_BLOCKS; ++j) {
-					q[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
-				}
-				dd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
-			}
-		}
-	}
-
-	// ---- 3. stage the activation slice in LDS: quants 16-byte aligned per half block, scales as fp32 ----
-	if constexpr (XF32) {
-#pragma unroll
-		for (int i = 0; i < XF_LOADS; ++i) {
-			const int v = lane + 64 * i;
-			uint16_t dh;
-			const uint32_t packed = quantize_block_lane(xf[i], &dh); // all lanes take part; lanes past the slice hold zeros
-			if (v < cnt * 32) {
-				*reinterpret_cast<uint32_t*>(xs_q + 4 * v) = packed; // block v/8 at 32*(v/8), dword v%8
-				if ((v & 7) == 0) {
-					xs_d[v >> 3] = half_bits_to_float(dh); // the fp16-rounded scale, exactly what a stored block would hold
-				}
-			}
-		}
-	} else {
-		// half-word hw of the raw stream is a scale (hw % 17 == 0) or a quant pair
-#pragma unroll
-		for (int i = 0; i < XQ_LOADS; ++i) {
-			const int v = lane + 64 * i;
-			if (v < cnt * 34) {
-#pragma unroll
-				for (int h = 0; h < 2; ++h) {
-					const int hw	   = 2 * v + h;
-					const int jj	   = hw / 17;
-					const int o		   = hw - 17 * jj;
-					const uint16_t val = static_cast<uint16_t>(h ? (xr[i] >> 16) : (xr[i] & 0xFFFFu));
-					if (o == 0) {
-						xs_d[jj] = half_bits_to_float(val);
-					} else {
-						*reinterpret_cast<uint16_t*>(xs_q + jj * QK + 2 * (o - 1)) = val;
-					}
-				}
-			}
-		}
-	}
-	__builtin_amdgcn_wave_barrier(); // wave-local hand-off: the same wave wrote and reads; the LDS counter wait orders it
-
-	if constexpr (DUMP == DUMP_X) {
-		// parity hook: what was staged, written back as packed blocks (the first strip of the launch covers all of K)
-		if (dump_this_strip) {
-			uint8_t* out = static_cast<uint8_t*>(dump) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * BLOCK_BYTES);
-			for (int jj = lane; jj < cnt * GROUP_BLOCKS; jj += 64) {
-				uint8_t* o						= out + jj * BLOCK_BYTES;
-				*reinterpret_cast<uint16_t*>(o) = float_to_half_bits(xs_d[jj]); // exact: the value came from fp16
-				for (int i = 0; i < 16; ++i) {
-					*reinterpret_cast<uint16_t*>(o + 2 + 2 * i) = *reinterpret_cast<const uint16_t*>(xs_q + jj * QK + 2 * i);
-				}
-			}
-		}
-		return 0.0f;
-	}
-
-	// ---- 4. dot products as the tiles land ----
-	float acc = 0.0f;
-#pragma unroll
-	for (int t = 0; t < TILES; ++t) {
-		if (t < cnt) {
-			const float dw[GROUP_BLOCKS] = { half_bits_to_float(static_cast<uint16_t>(dd[t].x & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].x >> 16)),
-				half_bits_to_float(static_cast<uint16_t>(dd[t].y & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].y >> 16)) };
-#pragma unroll
-			for (int j = 0; j < GROUP_BLOCKS; ++j) {
-				const int jj = t * GROUP_BLOCKS + j;
-				const v4i xv = *reinterpret_cast<const v4i*>(xs_q + jj * QK + 16 * half);
-				const int s	 = dot16(q[t][j], xv);
-				if constexpr (DUMP == DUMP_SUMS) {
-					const int full = s + __shfl_xor(s, 32);
-					if (half == 0 && row < N) {
-						static_cast<int32_t*>(dump)[static_cast<int64_t>(row) * (groups * GROUP_BLOCKS) + (gc * GROUP_BLOCKS + jj)] = full;
-					}
-				} else {
-					acc = fmaf(static_cast<float>(s), dw[j] * xs_d[jj], acc);
-				}
-			}
-		}
-	}
-	return acc;
-}
-
 template<int TILES, bool XF32, int DUMP, bool LOOP>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, float* __restrict__ partials,
 	unsigned* __restrict__ counters, int groups, int split_shift, int groups_per_slot, int groups_rem) {
@@ -316,7 +180,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	if (tid < STRIP_ROWS) {
 		__hip_atomic_store(&partials[(static_cast<int64_t>(gstrip) * splits + split) * STRIP_ROWS + tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 	}
-	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // s_waitcnt only: the stores above have completed
+	wait_stores_acknowledged();
 	__syncthreads();
 	if (tid == 0) {
 		const unsigned prev = __hip_atomic_fetch_add(&counters[gstrip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -349,15 +213,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	}
 }
 
-// Scratch of the K-split path: partial sums and arrival counters, one allocation per device, made on first use
-// and kept for the life of the process.  Calls that overlap on one GPU (different streams) and both split K race on it.
-constexpr int GEMV_MAX_SPLIT_UNITS	= 8192; // strips * splits when splits > 1
-constexpr int GEMV_MAX_SPLIT_STRIPS = 512;
-struct gemv_scratch {
-	float* partials	   = nullptr;
-	unsigned* counters = nullptr;
-};
-static hipError_t get_gemv_scratch(gemv_scratch* out) {
+hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	static std::mutex lock;
 	static gemv_scratch per_device[64];
 	int dev		 = 0;
@@ -372,46 +228,31 @@ static hipError_t get_gemv_scratch(gemv_scratch* out) {
 	gemv_scratch& sc = per_device[dev];
 	if (!sc.partials) {
 		void* p			   = nullptr;
-		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 4 + GEMV_MAX_SPLIT_STRIPS * 4;
+		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 4 + GEMV_MAX_SPLIT_STRIPS * 4 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * (8 + 1 + 1) * 4;
 		e				   = hipMalloc(&p, bytes);
 		if (e != hipSuccess) {
 			return e;
 		}
-		e = hipMemset(p, 0, bytes); // synchronous, once: counters start at zero and every launch leaves them at zero
+		e = hipMemset(p, 0, bytes); // synchronous, once: counters start at zero and every launch leaves them at zero; flags start at epoch 0
 		if (e != hipSuccess) {
 			(void)hipFree(p);
 			return e;
 		}
 		sc.partials = static_cast<float*>(p);
 		sc.counters = reinterpret_cast<unsigned*>(sc.partials + static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS);
+		sc.gate_up	= reinterpret_cast<float*>(sc.counters + GEMV_MAX_SPLIT_STRIPS);
+		sc.act_q	= reinterpret_cast<uint32_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
+		sc.act_d	= reinterpret_cast<float*>(sc.act_q + (FFN_MAX_HIDDEN / STRIP_ROWS) * 8);
+		sc.flags	= reinterpret_cast<unsigned*>(sc.act_d + FFN_MAX_HIDDEN / STRIP_ROWS);
+	}
+	if (next_epoch) {
+		++sc.epoch; // flags start at zero and the first epoch handed out is 1
+		if (sc.epoch == 0) {
+			++sc.epoch;
+		}
 	}
 	*out = sc;
 	return hipSuccess;
-}
-
-// How a tiled mat-vec launch is cut: `splits` workgroups per strip, each of 16 waves owning <= `tiles` groups.
-struct gemv_plan {
-	int strips, groups, splits, tiles;
-};
-static gemv_plan plan_gemv(int64_t total_strips, int64_t K) {
-	gemv_plan p;
-	p.strips	   = static_cast<int>(total_strips);
-	p.groups	   = static_cast<int>(K / GROUP_K);
-	p.splits	   = 1;
-	auto tiles_for = [&](int s) { return (p.groups + GEMV_WAVES * s - 1) / (GEMV_WAVES * s); };
-	// K goes over several workgroups only when it has to: the hand-off between workgroups costs 1-2 us, more than an
-	// idle half of the chip costs a matrix of a few MB.  So: split until a wave owns at most 4 groups (every load of the
-	// wave in flight at once), and, once splitting anyway, one step further to 2 groups per wave (measured best on the
-	// long-K down projections).
-	const bool room = p.strips <= GEMV_MAX_SPLIT_STRIPS;
-	while (tiles_for(p.splits) > 4 && room && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
-		p.splits *= 2;
-	}
-	if (p.splits > 1 && tiles_for(p.splits) > 2 && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
-		p.splits *= 2;
-	}
-	p.tiles = tiles_for(p.splits);
-	return p;
 }
 
 template<int TILES, bool XF32, bool LOOP> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, hipStream_t s) {

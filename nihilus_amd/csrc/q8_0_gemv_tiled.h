@@ -1,0 +1,245 @@
+// The streaming mat-vec on the tiled layout: pieces shared by the plain decode kernel and the fused FFN kernel.
+#pragma once
+#include "q8_0_device.h"
+
+namespace nh {
+
+constexpr int GEMV_WAVES = 16;
+
+struct gemv_segments {
+	const uint8_t* W[GEMV_MAX_SEGMENTS];
+	float* y[GEMV_MAX_SEGMENTS];
+	int rows[GEMV_MAX_SEGMENTS];
+	int strip_end[GEMV_MAX_SEGMENTS]; // running total of strips
+};
+
+enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
+
+// One chunk of a wave's K range: groups [gc, gc + cnt), cnt <= TILES, all wave-uniform (scalar registers).
+// xs_q / xs_d are this wave's private LDS slices.  Returns the lane's partial dot product over the chunk.
+//
+// XMODE says where the activation slice comes from:
+//   X_BLOCKS    packed Q8_0 blocks (xin), re-aligned into LDS;
+//   X_F32       fp32 values (xin), quantized on the spot;
+//   X_PUBLISHED quantized blocks that OTHER workgroups of the same launch produce (xin = quants, 8 dwords per block;
+//               xin2 = fp32 scales, one per block): the wave first puts all its weight loads in flight, then waits
+//               until the 4 * cnt blocks of its slice carry `epoch` in `flags` (one word per block), then reads them
+//               with device-scope loads.  The wait is bounded: after FLAG_SPIN_LIMIT polls the wave gives up and
+//               returns NaN, so the kernel always drains.
+enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2 };
+constexpr int FLAG_SPIN_LIMIT = 1 << 20;
+
+template<int TILES, int XMODE, int DUMP>
+__device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
+	int groups, int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2 = nullptr, const unsigned* __restrict__ flags = nullptr, unsigned epoch = 0) {
+	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
+	const int r	   = lane & 31;
+	const int half = lane >> 5;
+
+	// ---- 1. activation slice loads, issued first ----
+	constexpr int XQ_LOADS = (TILES * 34 + 63) / 64; // raw dwords of blocks [4*gc, 4*(gc+cnt)): 34 dwords per group
+	constexpr int XF_LOADS = (TILES * 32 + 63) / 64; // float4 per lane: 128 floats per group = 32 float4
+	uint32_t xr[XQ_LOADS];
+	float4 xf[XF_LOADS];
+	if constexpr (XMODE == X_F32) {
+		const float4* x4 = reinterpret_cast<const float4*>(static_cast<const float*>(xin) + static_cast<int64_t>(gc) * GROUP_K);
+#pragma unroll
+		for (int i = 0; i < XF_LOADS; ++i) {
+			const int v = lane + 64 * i; // float4 index in the slice; block = v / 8
+			xf[i]		= v < cnt * 32 ? x4[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+		}
+	} else if constexpr (XMODE == X_BLOCKS) {
+		const uint32_t* x_raw = reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(xin) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * BLOCK_BYTES));
+#pragma unroll
+		for (int i = 0; i < XQ_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			xr[i]		= v < cnt * 34 ? x_raw[v] : 0u;
+		}
+	}
+
+	// ---- 2. every weight byte of the chunk, in flight at once ----
+	v4i q[TILES][GROUP_BLOCKS];
+	v2u dd[TILES];
+	if constexpr (DUMP != DUMP_X) {
+		const uint8_t* macro0 = w_strip + static_cast<int64_t>(gc) * MACRO_BYTES;
+#pragma unroll
+		for (int t = 0; t < TILES; ++t) {
+			if (t < cnt) {
+				const uint8_t* macro = macro0 + t * MACRO_BYTES;
+#pragma unroll
+				for (int j = 0; j < GROUP_BLOCKS; ++j) {
+					q[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+				}
+				dd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+			}
+		}
+	}
+
+	// ---- 2b. the slice comes from this launch's own producers: wait for them, then fetch it ----
+	bool timed_out = false;
+	if constexpr (XMODE == X_PUBLISHED) {
+		const unsigned* f = flags + gc * GROUP_BLOCKS;
+		const int n_flags = cnt * GROUP_BLOCKS;
+		int spins		  = 0;
+		for (;;) {
+			const unsigned seen = lane < n_flags ? __hip_atomic_load(f + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : epoch;
+			if (__builtin_amdgcn_ballot_w64(seen != epoch) == 0) {
+				break;
+			}
+			if (++spins >= FLAG_SPIN_LIMIT) {
+				timed_out = true;
+				break;
+			}
+			__builtin_amdgcn_s_sleep(16);
+		}
+		asm volatile("" ::: "memory"); // the data loads below stay behind the flag loads above
+		// device-scope loads: the producers ran on other XCDs, whose L2 this one does not snoop
+		const uint32_t* pq = static_cast<const uint32_t*>(xin) + gc * (GROUP_BLOCKS * 8);
+		const float* pd	   = static_cast<const float*>(xin2) + gc * GROUP_BLOCKS;
+		constexpr int PQ_LOADS = (TILES * 32 + 63) / 64; // 32 dwords per group
+		uint32_t qv[PQ_LOADS];
+#pragma unroll
+		for (int i = 0; i < PQ_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			qv[i]		= v < cnt * 32 ? __hip_atomic_load(pq + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+		}
+		const float dv = lane < n_flags ? __hip_atomic_load(pd + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+#pragma unroll
+		for (int i = 0; i < PQ_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			if (v < cnt * 32) {
+				*reinterpret_cast<uint32_t*>(xs_q + 4 * v) = qv[i]; // block v/8 at 32*(v/8), dword v%8
+			}
+		}
+		if (lane < n_flags) {
+			xs_d[lane] = dv;
+		}
+	}
+
+	// ---- 3. stage the activation slice in LDS: quants 16-byte aligned per half block, scales as fp32 ----
+	if constexpr (XF32) {
+#pragma unroll
+		for (int i = 0; i < XF_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			uint16_t dh;
+			const uint32_t packed = quantize_block_lane(xf[i], &dh); // all lanes take part; lanes past the slice hold zeros
+			if (v < cnt * 32) {
+				*reinterpret_cast<uint32_t*>(xs_q + 4 * v) = packed; // block v/8 at 32*(v/8), dword v%8
+				if ((v & 7) == 0) {
+					xs_d[v >> 3] = half_bits_to_float(dh); // the fp16-rounded scale, exactly what a stored block would hold
+				}
+			}
+		}
+	} else if constexpr (XMODE == X_BLOCKS) {
+		// half-word hw of the raw stream is a scale (hw % 17 == 0) or a quant pair
+#pragma unroll
+		for (int i = 0; i < XQ_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			if (v < cnt * 34) {
+#pragma unroll
+				for (int h = 0; h < 2; ++h) {
+					const int hw	   = 2 * v + h;
+					const int jj	   = hw / 17;
+					const int o		   = hw - 17 * jj;
+					const uint16_t val = static_cast<uint16_t>(h ? (xr[i] >> 16) : (xr[i] & 0xFFFFu));
+					if (o == 0) {
+						xs_d[jj] = half_bits_to_float(val);
+					} else {
+						*reinterpret_cast<uint16_t*>(xs_q + jj * QK + 2 * (o - 1)) = val;
+					}
+				}
+			}
+		}
+	}
+	__builtin_amdgcn_wave_barrier(); // wave-local hand-off: the same wave wrote and reads; the LDS counter wait orders it
+
+	if constexpr (DUMP == DUMP_X) {
+		// parity hook: what was staged, written back as packed blocks (the first strip of the launch covers all of K)
+		if (dump_this_strip) {
+			uint8_t* out = static_cast<uint8_t*>(dump) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * BLOCK_BYTES);
+			for (int jj = lane; jj < cnt * GROUP_BLOCKS; jj += 64) {
+				uint8_t* o						= out + jj * BLOCK_BYTES;
+				*reinterpret_cast<uint16_t*>(o) = float_to_half_bits(xs_d[jj]); // exact: the value came from fp16
+				for (int i = 0; i < 16; ++i) {
+					*reinterpret_cast<uint16_t*>(o + 2 + 2 * i) = *reinterpret_cast<const uint16_t*>(xs_q + jj * QK + 2 * i);
+				}
+			}
+		}
+		return 0.0f;
+	}
+
+	// ---- 4. dot products as the tiles land ----
+	float acc = 0.0f;
+#pragma unroll
+	for (int t = 0; t < TILES; ++t) {
+		if (t < cnt) {
+			const float dw[GROUP_BLOCKS] = { half_bits_to_float(static_cast<uint16_t>(dd[t].x & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].x >> 16)),
+				half_bits_to_float(static_cast<uint16_t>(dd[t].y & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].y >> 16)) };
+#pragma unroll
+			for (int j = 0; j < GROUP_BLOCKS; ++j) {
+				const int jj = t * GROUP_BLOCKS + j;
+				const v4i xv = *reinterpret_cast<const v4i*>(xs_q + jj * QK + 16 * half);
+				const int s	 = dot16(q[t][j], xv);
+				if constexpr (DUMP == DUMP_SUMS) {
+					const int full = s + __shfl_xor(s, 32);
+					if (half == 0 && row < N) {
+						static_cast<int32_t*>(dump)[static_cast<int64_t>(row) * (groups * GROUP_BLOCKS) + (gc * GROUP_BLOCKS + jj)] = full;
+					}
+				} else {
+					acc = fmaf(static_cast<float>(s), dw[j] * xs_d[jj], acc);
+				}
+			}
+		}
+	}
+	if constexpr (XMODE == X_PUBLISHED) {
+		if (timed_out) {
+			acc = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output
+		}
+	}
+	return acc;
+}
+
+// Scratch of the K-split path (partial sums and arrival counters) and of the fused FFN launch (the gate and up
+// projections' outputs and one "published" word per producer strip): one allocation per device, made on first use and
+// kept for the life of the process.  Calls that overlap on one GPU (different streams) and both use it race on it.
+constexpr int GEMV_MAX_SPLIT_UNITS	= 8192; // strips * splits when splits > 1
+constexpr int GEMV_MAX_SPLIT_STRIPS = 512;
+constexpr int FFN_MAX_HIDDEN		= 65536; // rows of the gate / up projections in a fused FFN launch
+struct gemv_scratch {
+	float* partials	   = nullptr;
+	unsigned* counters = nullptr;
+	float* gate_up	   = nullptr; // [2][FFN_MAX_HIDDEN]: the gate and up outputs (kept for inspection only)
+	uint32_t* act_q	   = nullptr; // [FFN_MAX_HIDDEN / 32][8]: the quantized activation of the down projection, 8 dwords per block
+	float* act_d	   = nullptr; // [FFN_MAX_HIDDEN / 32]: its scales (the fp16-rounded value, widened)
+	unsigned* flags	   = nullptr; // [FFN_MAX_HIDDEN / 32]: the epoch of the launch that last published the block
+	unsigned epoch	   = 0; // with next_epoch = true: a value no earlier launch on this device has used
+};
+hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch = false);
+
+// How a tiled mat-vec launch is cut: `splits` workgroups per strip, each of 16 waves owning <= `tiles` groups.
+struct gemv_plan {
+	int strips, groups, splits, tiles;
+};
+inline gemv_plan plan_gemv(int64_t total_strips, int64_t K) {
+	gemv_plan p;
+	p.strips	   = static_cast<int>(total_strips);
+	p.groups	   = static_cast<int>(K / GROUP_K);
+	p.splits	   = 1;
+	auto tiles_for = [&](int s) { return (p.groups + GEMV_WAVES * s - 1) / (GEMV_WAVES * s); };
+	// K goes over several workgroups only when it has to: the hand-off between workgroups costs 1-2 us, more than an
+	// idle half of the chip costs a matrix of a few MB.  So: split until a wave owns at most 4 groups (every load of the
+	// wave in flight at once), and, once splitting anyway, one step further to 2 groups per wave (measured best on the
+	// long-K down projections).
+	const bool room = p.strips <= GEMV_MAX_SPLIT_STRIPS;
+	while (tiles_for(p.splits) > 4 && room && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
+		p.splits *= 2;
+	}
+	if (p.splits > 1 && tiles_for(p.splits) > 2 && p.strips * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
+		p.splits *= 2;
+	}
+	p.tiles = tiles_for(p.splits);
+	return p;
+}
+
+
+} // namespace nh

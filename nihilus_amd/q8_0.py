@@ -101,6 +101,30 @@ def get_rows(w: torch.Tensor, ids: torch.Tensor, n_rows: int, k: int, tiled: boo
     return (out, int(bad.item())) if count_invalid else out
 
 
+def ffn(w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, x: torch.Tensor, n_ff: int, k: int, n_out: int, residual: torch.Tensor | None = None) -> torch.Tensor:
+    """Decode-time FFN in one launch: W_down . Q(silu(W_gate . Q(x)) * (W_up . Q(x))) (+ residual); weights tiled, x fp32 [k]."""
+    w_gate, w_up, w_down = _dev(w_gate, torch.uint8, "w_gate"), _dev(w_up, torch.uint8, "w_up"), _dev(w_down, torch.uint8, "w_down")
+    x = _dev(x, torch.float32, "x")
+    if w_gate.numel() != tiled_bytes(n_ff, k) or w_up.numel() != tiled_bytes(n_ff, k) or w_down.numel() != tiled_bytes(n_out, n_ff) or x.numel() != k:
+        raise ValueError("operand sizes do not match n_ff x k / n_out x n_ff")
+    if residual is not None:
+        residual = _dev(residual, torch.float32, "residual")
+        if residual.numel() != n_out:
+            raise ValueError("residual must hold n_out values")
+    y = torch.empty(n_out, dtype=torch.float32, device=x.device)
+    _lib.check("nh_q8_0_ffn_f32", _lib.lib().nh_q8_0_ffn_f32(w_gate.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), x.data_ptr(),
+                                                           residual.data_ptr() if residual is not None else None, y.data_ptr(), n_ff, k, n_out, _stream()))
+    return y
+
+
+def debug_ffn_gate_up(n_ff: int):
+    """The gate and up outputs (fp32 [n_ff] each) of the last ffn() on this device."""
+    g = torch.empty(n_ff, dtype=torch.float32, device="cuda")
+    u = torch.empty(n_ff, dtype=torch.float32, device="cuda")
+    _lib.check("nh_q8_0_debug_ffn_gate_up", _lib.lib().nh_q8_0_debug_ffn_gate_up(g.data_ptr(), u.data_ptr(), n_ff, _stream()))
+    return g, u
+
+
 def gemv(w: torch.Tensor, xq_blocks: torch.Tensor, n: int, k: int, tiled: bool) -> torch.Tensor:
     w, xq_blocks = _dev(w, torch.uint8, "w"), _dev(xq_blocks, torch.uint8, "xq_blocks")
     if w.numel() != (tiled_bytes(n, k) if tiled else blocks_bytes(n, k)) or xq_blocks.numel() != blocks_bytes(1, k):
