@@ -45,7 +45,10 @@ typedef enum nh_status {
 	NH_ERR_SHAPE	   = -3, /* negative size, K % 32 != 0, or K % 128 != 0 for a tiled operand */
 	NH_ERR_NO_DEVICE   = -4, /* no gfx950 device visible */
 	NH_ERR_TOO_LARGE   = -5, /* a dimension exceeds what the launch grid or 32-bit tile indices hold */
-	NH_ERR_ARGUMENT	   = -6 /* any other invalid argument */
+	NH_ERR_ARGUMENT	   = -6, /* any other invalid argument */
+	NH_ERR_IO		   = -7, /* a file could not be opened or mapped */
+	NH_ERR_FORMAT	   = -8, /* a file is not what its reader accepts */
+	NH_ERR_NOT_FOUND   = -9 /* no tensor or metadata key of that name */
 } nh_status;
 
 /* Library / device ------------------------------------------------------------------------------ */

@@ -10,7 +10,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libnihilus_q8_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-SOURCES = ["q8_0_abi.hip", "q8_0_quantize.hip", "q8_0_layout.hip", "q8_0_get_rows.hip", "q8_0_gemv.hip", "q8_0_ffn.hip", "q8_0_gemm.hip", "q8_0_gemm_skinny.hip", "q8_0_profile.hip"]
+SOURCES = ["q8_0_abi.hip", "q8_0_quantize.hip", "q8_0_layout.hip", "q8_0_get_rows.hip", "q8_0_gemv.hip", "q8_0_ffn.hip", "q8_0_gemm.hip", "q8_0_gemm_skinny.hip", "q8_0_profile.hip", "gguf_q8_0.cpp"]
 
 # -packed-fp32-ops off: v_pk_{add,mul,fma}_f32 are kept out of the generated code on purpose.
 # No -ffast-math: the quantizer needs IEEE divide, unfused multiply and round-half-even.
@@ -40,7 +40,8 @@ def hipcc() -> str:
 
 def build_library(verbose: bool = False, extra_flags: list[str] | None = None) -> str:
     """Compile every HIP source into one shared library next to this file. Always recompiles."""
-    cmd = [hipcc(), *HIPCC_FLAGS, *(extra_flags or []), "-o", LIB_PATH, *[os.path.join(CSRC, s) for s in SOURCES]]
+    include = os.path.join(os.path.dirname(PKG_DIR), "include")
+    cmd = [hipcc(), *HIPCC_FLAGS, "-I", include, *(extra_flags or []), "-o", LIB_PATH, *[os.path.join(CSRC, s) for s in SOURCES]]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature name and says so once per source: not an error
     noise = "is not a recognized feature for this target"

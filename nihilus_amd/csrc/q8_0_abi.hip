@@ -97,6 +97,12 @@ const char* nh_status_string(int status) {
 			return "dimension too large";
 		case NH_ERR_ARGUMENT:
 			return "invalid argument";
+		case NH_ERR_IO:
+			return "file could not be opened or mapped";
+		case NH_ERR_FORMAT:
+			return "file format not accepted";
+		case NH_ERR_NOT_FOUND:
+			return "name not found";
 		default:
 			return status > 0 ? hipGetErrorString(static_cast<hipError_t>(status)) : "unknown status";
 	}
