@@ -143,7 +143,7 @@ def main() -> int:
         for i in range(start, start + count):
             if fused:
                 g, u, d = ptrs[i % L]
-                rc = ffn(g, u, d, x_ptr, None, y_ptr, FFN, HIDDEN, HIDDEN, stream)
+                rc = ffn(g, u, d, x_ptr, None, 0.0, None, y_ptr, FFN, HIDDEN, HIDDEN, stream)
             else:
                 rc = batch(op_lists[i % L], 3, ws_ptr, ws_n, stream)
             if rc != 0:

@@ -218,6 +218,17 @@ namespace nihilus {
 		static constexpr uint64_t ne01 = input_type01::get_array()[1]; // N
 		static_assert(ne00 % 128 == 0, "the tiled weight layout needs K to be a multiple of 128");
 
+		// The same with the rms_norm and mul nodes that precede the projection folded in: activation is the un-normalised
+		// row, norm_weight the fp32 [K] norm weight, eps the model's layer_norm_rms_epsilon (infra/core_traits.hpp:570-576).
+		static void impl(core_traits_type& output, const void* weight_tiled, const float* activation, const float* norm_weight, float eps, void* stream = nullptr) {
+			float* y		= output.template get_data<float>();
+			const int64_t n = ne01;
+			amd_detail::check<config_type>(nh_q8_0_gemv_tiled_multi_norm_f32(&weight_tiled, &y, &n, 1, activation, norm_weight, eps, ne00, stream), "eval_time norm + mat-vec");
+			if constexpr (config_type::synchronous) {
+				amd_detail::check<config_type>(nh_stream_sync(stream), "stream sync");
+			}
+		}
+
 		// weight: device pointer to the tiled matrix; activation: fp32 [K]; output: fp32 [N]; stream may be null
 		static void impl(core_traits_type& output, const void* weight_tiled, const float* activation, void* stream = nullptr) {
 			amd_detail::check<config_type>(nh_q8_0_gemv_tiled_f32(weight_tiled, activation, output.template get_data<float>(), ne01, ne00, stream), "eval_time mat-vec");

@@ -89,6 +89,16 @@ int nh_q8_0_quantize_tiled(const float* x, void* xq_tiled, int64_t M, int64_t K,
 int nh_q8_0_silu_mul_quantize(const float* gate, const float* up, void* xq_blocks, int64_t M, int64_t K, void* stream);
 int nh_q8_0_silu_mul_quantize_tiled(const float* gate, const float* up, void* xq_tiled, int64_t M, int64_t K, void* stream);
 
+/* RMS norm * weight fused into the quantizer: xq[m] = quantize_row_q8_0((x[m] * scale_m) * norm_weight),
+ * scale_m = 1 / sqrt(mean(x[m]^2) + eps).  Stands for the rms_norm -> mul -> activation operand chain in front of
+ * the q/k/v, gate/up and output projections (infra/core_traits.hpp:570-576, :971-974, :1186-1190; dead fused attempt
+ * cpu/avx_2.hpp:5331-5384, whose sqrtf_fast is an exact square root on one ISA and a bit trick on another,
+ * cpu/common.hpp:310/448: here it is the IEEE square root and divide).  The sum of squares is taken in a fixed order
+ * (see the CPU checker's nho_rms_norm_scale for the same order), so the quantized bytes are reproducible.
+ * x: fp32 [M][K]; norm_weight: fp32 [K]; 0 <= eps < 1; K % 128 == 0 for both output layouts. */
+int nh_q8_0_rms_norm_quantize(const float* x, const float* norm_weight, float eps, void* xq_blocks, int64_t M, int64_t K, void* stream);
+int nh_q8_0_rms_norm_quantize_tiled(const float* x, const float* norm_weight, float eps, void* xq_tiled, int64_t M, int64_t K, void* stream);
+
 /* Layout conversion ---------------------------------------------------------------------------- */
 
 /* Bytes of a [rows x K] matrix: blocks = rows*(K/32)*34 (type_traits<block_q8_0>::total_byte_size,
@@ -128,19 +138,26 @@ int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_
 /* The same for up to 3 weight matrices that share K and x (q/k/v, gate/up: infra/core_traits.hpp:575-594, :976-986)
  * as ONE launch: y[i] = W_tiled[i] . quantize(x), i < count.  host_* arrays are host memory, read before return. */
 int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream);
+/* The same with the RMS norm in front: y[i] = W_tiled[i] . quantize((x * scale) * norm_weight), scale = 1 / sqrt(mean(x^2) + eps),
+ * all inside the one launch (the values of nh_q8_0_rms_norm_quantize + nh_q8_0_gemv_tiled).  This is the decode-time
+ * rms_norm -> mul -> q/k/v (or gate/up, or output) group of the reference's mega cores (infra/core_traits.hpp:570-594). */
+int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, const float* norm_weight, float eps,
+	int64_t K, void* stream);
 
-/* The decode-time FFN as one launch:  y = W_down . Q(silu(W_gate . Q(x)) * (W_up . Q(x))) [+ residual],  Q = quantize_row_q8_0.
+/* The decode-time FFN as one launch:  y = W_down . Q(silu(W_gate . Q(n)) * (W_up . Q(n))) [+ residual],  Q = quantize_row_q8_0,
+ * n = x, or with norm_weight != NULL n = (x * scale) * norm_weight (RMS norm as in nh_q8_0_rms_norm_quantize).
  * Stands for the eval_time body of the reference's mega_ffn core: ffn_gate and ffn_up mul_mat, silu, mul, ffn_down
  * mul_mat, residual add (infra/core_traits.hpp:971-995; the GPU dispatcher that would hold it is empty,
- * cuda/cuda_12.hpp:806-916).  Same arithmetic, bit for bit, as nh_q8_0_gemv_tiled_multi_f32 (gate, up) followed by
- * nh_q8_0_silu_mul_quantize and nh_q8_0_gemv_tiled (down): the down projection's workgroups ride in the same grid
- * and start streaming their weights while gate/up are still running.
+ * cuda/cuda_12.hpp:806-916).  Same arithmetic as nh_q8_0_gemv_tiled_multi_[norm_]f32 (gate, up) followed by
+ * nh_q8_0_silu_mul_quantize and nh_q8_0_gemv_tiled (down), with K cut differently (last-bit differences in the fp32
+ * sums): the down projection's workgroups ride in the same grid and start streaming their weights while gate/up are
+ * still running.
  * W_gate, W_up: [N_ff x K] tiled; W_down: [N_out x N_ff] tiled; x: fp32 [K]; residual: fp32 [N_out] or NULL;
  * y: fp32 [N_out] (may alias residual).  K % 128 == 0, N_ff % 128 == 0, N_ff <= NH_Q8_0_FFN_MAX_HIDDEN.
  * Uses the library's per-device scratch: two such calls must not overlap on one GPU. */
 #define NH_Q8_0_FFN_MAX_HIDDEN 65536
-int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* residual, float* y, int64_t N_ff, int64_t K, int64_t N_out,
-	void* stream);
+int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* norm_weight, float eps, const float* residual, float* y,
+	int64_t N_ff, int64_t K, int64_t N_out, void* stream);
 
 /* Mat-mat (prefill, prompt_eval_time) ----------------------------------------------------------- */
 
@@ -196,11 +213,13 @@ int nh_profile_end(double* host_total_ms, int64_t* host_launches, double* host_m
 int nh_q8_0_debug_block_sums(const void* W, const void* Aq, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream);
 
 /* What the fused mat-vec stages for x: runs the fused kernel's own quantize-and-stage code on fp32 x [K] and writes
- * the staged row back as K/32 packed blocks, to be compared byte for byte with nh_q8_0_quantize. K % 128 == 0. */
+ * the staged row back as K/32 packed blocks, to be compared byte for byte with nh_q8_0_quantize (or, with a norm
+ * weight, with nh_q8_0_rms_norm_quantize). K % 128 == 0. */
+int nh_q8_0_debug_fused_quantize(const float* x, void* xq_blocks_out, int64_t K, void* stream);
+int nh_q8_0_debug_fused_norm_quantize(const float* x, const float* norm_weight, float eps, void* xq_blocks_out, int64_t K, void* stream);
 /* The gate and up projections' fp32 outputs of the last nh_q8_0_ffn_f32 on this device (they never leave the
  * library otherwise), copied out for comparison. */
 int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void* stream);
-int nh_q8_0_debug_fused_quantize(const float* x, void* xq_blocks_out, int64_t K, void* stream);
 
 /* Synthetic inputs (benchmark / test utility) --------------------------------------------------- */
 

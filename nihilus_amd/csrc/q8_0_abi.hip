@@ -282,8 +282,8 @@ int nh_q8_0_get_rows_tiled(const void* W_tiled, const int32_t* ids, float* out, 
 	return get_rows_common(W_tiled, ids, out, invalid_count, n_tokens, n_rows, K, true, stream);
 }
 
-int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* residual, float* y, int64_t N_ff, int64_t K, int64_t N_out,
-	void* stream) {
+int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* norm_weight, float eps, const float* residual, float* y,
+	int64_t N_ff, int64_t K, int64_t N_out, void* stream) {
 	NH_TRY(check_shape(N_ff, 0, K, true)); // gate, up: [N_ff x K]
 	NH_TRY(check_shape(N_out, 0, N_ff, true)); // down: [N_out x N_ff]
 	NH_REQUIRE(N_ff <= NH_Q8_0_FFN_MAX_HIDDEN, NH_ERR_TOO_LARGE);
@@ -291,13 +291,14 @@ int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void
 		return NH_OK;
 	}
 	NH_REQUIRE(y, NH_ERR_NULL_POINTER);
-	NH_REQUIRE(aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(aligned16(y) && aligned16(residual) && aligned16(norm_weight), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(!norm_weight || (eps >= 0.0f && eps < 1.0f), NH_ERR_ARGUMENT);
 	if (N_ff > 0 && K > 0) {
 		NH_REQUIRE(W_gate_tiled && W_up_tiled && W_down_tiled && x, NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(W_gate_tiled) && aligned16(W_up_tiled) && aligned16(W_down_tiled) && aligned16(x), NH_ERR_ALIGNMENT);
 	}
 	NH_TRY(require_device());
-	return from_hip(nh::launch_ffn_decode(W_gate_tiled, W_up_tiled, W_down_tiled, x, residual, y, N_ff, K, N_out, as_stream(stream)));
+	return from_hip(nh::launch_ffn_decode(W_gate_tiled, W_up_tiled, W_down_tiled, x, norm_weight, eps, residual, y, N_ff, K, N_out, as_stream(stream)));
 }
 
 int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void* stream) {
@@ -335,7 +336,8 @@ int nh_q8_0_gemv_tiled(const void* W_tiled, const void* xq_blocks, float* y, int
 	return gemv_common(W_tiled, xq_blocks, y, N, K, true, stream);
 }
 
-int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream) {
+static int gemv_multi_common(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, const float* norm_weight, float eps, int64_t K,
+	void* stream) {
 	NH_REQUIRE(count >= 0 && count <= nh::GEMV_MAX_SEGMENTS, NH_ERR_ARGUMENT);
 	if (count == 0) {
 		return NH_OK;
@@ -365,23 +367,59 @@ int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* 
 		NH_REQUIRE(x, NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(x), NH_ERR_ALIGNMENT);
 	}
+	NH_REQUIRE(aligned16(norm_weight), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(!norm_weight || (eps >= 0.0f && eps < 1.0f), NH_ERR_ARGUMENT);
 	NH_TRY(require_device());
-	return from_hip(nh::launch_gemv_tiled_multi(host_W_tiled, host_y, host_N, static_cast<int>(count), x, true, K, as_stream(stream)));
+	return from_hip(nh::launch_gemv_tiled_multi(host_W_tiled, host_y, host_N, static_cast<int>(count), x, true, K, as_stream(stream), norm_weight, eps));
+}
+
+int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream) {
+	return gemv_multi_common(host_W_tiled, host_y, host_N, count, x, nullptr, 0.0f, K, stream);
+}
+
+int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, const float* norm_weight, float eps,
+	int64_t K, void* stream) {
+	NH_REQUIRE(norm_weight || K == 0 || count == 0, NH_ERR_NULL_POINTER);
+	return gemv_multi_common(host_W_tiled, host_y, host_N, count, x, norm_weight, eps, K, stream);
 }
 
 int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream) {
 	return nh_q8_0_gemv_tiled_multi_f32(&W_tiled, &y, &N, 1, x, K, stream);
 }
 
-int nh_q8_0_debug_fused_quantize(const float* x, void* xq_blocks_out, int64_t K, void* stream) {
+int nh_q8_0_debug_fused_norm_quantize(const float* x, const float* norm_weight, float eps, void* xq_blocks_out, int64_t K, void* stream) {
 	NH_TRY(check_shape(1, 0, K, true));
 	if (K == 0) {
 		return NH_OK;
 	}
 	NH_REQUIRE(x && xq_blocks_out, NH_ERR_NULL_POINTER);
-	NH_REQUIRE(aligned16(x) && aligned16(xq_blocks_out), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(aligned16(x) && aligned16(xq_blocks_out) && aligned16(norm_weight), NH_ERR_ALIGNMENT);
 	NH_TRY(require_device());
-	return from_hip(nh::launch_gemv_dump_staged_x(x, xq_blocks_out, K, as_stream(stream)));
+	return from_hip(nh::launch_gemv_dump_staged_x(x, xq_blocks_out, K, as_stream(stream), norm_weight, eps));
+}
+
+int nh_q8_0_debug_fused_quantize(const float* x, void* xq_blocks_out, int64_t K, void* stream) {
+	return nh_q8_0_debug_fused_norm_quantize(x, nullptr, 0.0f, xq_blocks_out, K, stream);
+}
+
+static int rms_norm_quantize_common(const float* x, const float* norm_weight, float eps, void* xq, int64_t M, int64_t K, bool tiled, void* stream) {
+	NH_TRY(check_shape(M, 0, K, true)); // the fixed order of the sum of squares is defined on 128-value groups, whatever the output layout
+	if (M == 0 || K == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(x && norm_weight && xq, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(x) && aligned16(norm_weight) && aligned16(xq), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(eps >= 0.0f && eps < 1.0f, NH_ERR_ARGUMENT);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_rms_norm_quantize(x, norm_weight, eps, xq, M, K, tiled, as_stream(stream)));
+}
+
+int nh_q8_0_rms_norm_quantize(const float* x, const float* norm_weight, float eps, void* xq_blocks, int64_t M, int64_t K, void* stream) {
+	return rms_norm_quantize_common(x, norm_weight, eps, xq_blocks, M, K, false, stream);
+}
+
+int nh_q8_0_rms_norm_quantize_tiled(const float* x, const float* norm_weight, float eps, void* xq_tiled, int64_t M, int64_t K, void* stream) {
+	return rms_norm_quantize_common(x, norm_weight, eps, xq_tiled, M, K, true, stream);
 }
 
 static int gemm_common(const void* W, const void* A, float* C, int64_t M, int64_t N, int64_t K, bool tiled, void* stream) {

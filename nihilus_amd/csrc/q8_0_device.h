@@ -103,6 +103,70 @@ __device__ __forceinline__ float4 silu_mul4(float4 g, float4 u) {
 	return make_float4(silu_mul(g.x, u.x), silu_mul(g.y, u.y), silu_mul(g.z, u.z), silu_mul(g.w, u.w));
 }
 
+// RMS norm of a row, as a fixed order of fp32 operations over a 1024-thread workgroup (16 waves), restated by the CPU
+// checker so that the normalised, quantized row is reproducible bit for bit:
+//   runs:      the row's G = K / 128 groups are cut into 16 contiguous runs, run w = groups [w*q + min(w, r), ...) with
+//              q = G / 16, r = G % 16 and the first r runs one group longer (the cut of an unsplit mat-vec launch);
+//   lane l of wave w:  p = sum over the float4s l, l + 64, l + 128, ... of run w of x.x^2 + x.y^2 + x.z^2 + x.w^2,
+//              each term folded in by fma, float4s in ascending order;
+//   wave:      xor-butterfly over lane distances 32, 16, 8, 4, 2, 1 (every lane ends with the same value);
+//   workgroup: the 16 wave sums added in wave order;
+//   scale = 1 / sqrt(sum / K + eps) with IEEE divide and square root (the model's rms_norm; the reference's
+//   sqrtf_fast, cpu/common.hpp:310/448, is an exact sqrt on one ISA and a bit trick on another, cpu/avx_2.hpp:5382-5384);
+//   y_i = (x_i * scale) * w_i: the rms_norm node, then the mul node with the norm weight (infra/core_traits.hpp:570-573).
+__device__ __forceinline__ float sumsq_fold(float p, float4 v) {
+	p = fmaf(v.x, v.x, p);
+	p = fmaf(v.y, v.y, p);
+	p = fmaf(v.z, v.z, p);
+	return fmaf(v.w, v.w, p);
+}
+__device__ __forceinline__ float wave_sum_butterfly(float p) {
+#pragma unroll
+	for (int off = 32; off >= 1; off >>= 1) {
+		p = __fadd_rn(p, __shfl_xor(p, off));
+	}
+	return p;
+}
+// lane's share of run `wave` of a row of `groups` 128-value groups (K % 128 == 0)
+__device__ __forceinline__ float rms_run_sumsq(const float* x, int groups, int wave, int lane) {
+	const int q	 = groups / 16, r = groups % 16;
+	const int g0 = wave * q + min(wave, r);
+	const int n4 = (q + (wave < r ? 1 : 0)) * 32; // float4s in the run
+	const float4* x4 = reinterpret_cast<const float4*>(x) + g0 * 32;
+	float p			 = 0.0f;
+	for (int j = lane; j < n4; j += 64) {
+		p = sumsq_fold(p, x4[j]);
+	}
+	return p;
+}
+// red: 16 floats of LDS.  Contains a workgroup barrier: every thread of the 1024 must call it.
+__device__ __forceinline__ float rms_scale_workgroup(float p, float* red, int wave, int lane, int K, float eps) {
+	p = wave_sum_butterfly(p);
+	if (lane == 0) {
+		red[wave] = p;
+	}
+	__syncthreads();
+	float sum = red[0];
+#pragma unroll
+	for (int w = 1; w < 16; ++w) {
+		sum = __fadd_rn(sum, red[w]);
+	}
+	return __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(sum, static_cast<float>(K)), eps))); // sqrtf is correctly rounded; __fsqrt_rn maps to the 1-ulp native one
+}
+__device__ __forceinline__ float4 norm_mul4(float4 x, float scale, float4 w) {
+	return make_float4(__fmul_rn(__fmul_rn(x.x, scale), w.x), __fmul_rn(__fmul_rn(x.y, scale), w.y), __fmul_rn(__fmul_rn(x.z, scale), w.z), __fmul_rn(__fmul_rn(x.w, scale), w.w));
+}
+
+// 16 bytes per lane from global memory straight into LDS (lane l of the wave lands at lds_dst + 16 * l), no destination
+// registers.  Written as inline assembly rather than through the compiler's builtin because the compiler, not able
+// to tell which later LDS access such a transfer feeds, waits for ALL outstanding loads (the whole weight stream)
+// at the next LDS access.  The caller orders its LDS reads behind the transfer itself: loads complete in issue order,
+// so waiting for any register load issued after this one is enough.  lds_dst must be wave-uniform.
+__device__ __forceinline__ void load_global_to_lds_b128(const void* src, void* lds_dst) {
+	const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)(static_cast<char*>(lds_dst))));
+	asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory", "m0");
+}
+
 // Blocks the wave until every memory operation it has issued, stores included, has been acknowledged.  Placed
 // between device-scope (write-through) stores of data and the device-scope store or atomic that tells another
 // workgroup the data is there: a workgroup-scope release fence does not wait for the stores on this target, and an
@@ -139,6 +203,7 @@ inline hipError_t launch_kernel(int kind, Kernel kernel, dim3 grid, dim3 block, 
 // ---- launch functions (defined one per .hip file, called from q8_0_abi.hip after argument checks) ----
 
 hipError_t launch_quantize(const float* x, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s);
+hipError_t launch_rms_norm_quantize(const float* x, const float* norm_w, float eps, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s);
 hipError_t launch_silu_mul_quantize(const float* gate, const float* up, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s);
 hipError_t launch_tile(const void* blocks, void* tiled, int64_t rows, int64_t K, hipStream_t s);
 hipError_t launch_untile(const void* tiled, void* blocks, int64_t rows, int64_t K, hipStream_t s);
@@ -151,12 +216,13 @@ hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* 
 // one launch computes y[i] = W[i] . x for all of them.  x is either one row of packed blocks (x_is_f32 = false)
 // or the fp32 activations themselves, quantized inside the kernel (x_is_f32 = true).
 constexpr int GEMV_MAX_SEGMENTS = 3;
-hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s);
+hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s,
+	const float* norm_w = nullptr, float norm_eps = 0.0f);
 // Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
-hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* residual, float* y, int64_t n_ff, int64_t K, int64_t n_out,
-	hipStream_t s);
+hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* norm_w, float norm_eps, const float* residual, float* y, int64_t n_ff,
+	int64_t K, int64_t n_out, hipStream_t s);
 hipError_t copy_ffn_gate_up(float* gate_out, float* up_out, int64_t n_ff, hipStream_t s);
-hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s);
+hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w = nullptr, float norm_eps = 0.0f);
 hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s);
 // Tiled operands, M <= GEMM_SKINNY_MAX_M: the HBM-streaming MFMA kernel for batched decode (q8_0_gemm_skinny.hip).
 constexpr int64_t GEMM_SKINNY_MAX_M = 64;

@@ -29,6 +29,8 @@ struct ffn_args {
 	const uint8_t* w_up;
 	const uint8_t* w_down;
 	const float* x; // [K]
+	const float* norm_w; // [K] or null: RMS norm * weight applied to x in front of the gate/up quantizer
+	float norm_eps;
 	const float* residual; // [n_out] or null
 	float* y; // [n_out]
 	float* gate_up; // scratch: g at [0, n_ff), u at [FFN_MAX_HIDDEN, FFN_MAX_HIDDEN + n_ff), kept for inspection
@@ -45,7 +47,7 @@ struct ffn_args {
 	int split_shift, c_per_slot, c_rem; // a consumer strip's K range over splits * 16 waves
 };
 
-template<int TILES, bool LOOP> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
+template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K];
 	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
 	__shared__ float red[GEMV_WAVES][64];
@@ -59,6 +61,14 @@ template<int TILES, bool LOOP> __global__ __launch_bounds__(GEMV_WAVES * 64) voi
 	if (wg < a.producers) {
 		// ---- rows [32 * wg, 32 * wg + 32) of gate (waves 0-7) and of up (waves 8-15) -> activation block wg ----
 		__shared__ __align__(16) float act_f[STRIP_ROWS];
+		__shared__ float norm_red[16];
+		__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1];
+		gemv_norm norm_state;
+		gemv_norm* norm = nullptr;
+		if constexpr (NORM) { // eight waves per matrix here: the slices are not the sixteen runs of the fixed order, so the scale comes first
+			gemv_norm_begin(norm_state, a.x, a.norm_w, xs_w[NORM ? wave : 0], norm_red, a.norm_eps, a.groups_p * GROUP_K, lane, wave, false);
+			norm = &norm_state;
+		}
 		const int matrix	   = wave >> 3;
 		const int slot		   = wave & 7;
 		const int strip		   = wg;
@@ -68,10 +78,11 @@ template<int TILES, bool LOOP> __global__ __launch_bounds__(GEMV_WAVES * 64) voi
 		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
 		float acc			   = 0.0f;
 		if constexpr (!LOOP) {
-			acc = gemv_chunk<TILES, X_F32, DUMP_NONE>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false);
+			acc = gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, nullptr, nullptr, 0, norm);
 		} else {
 			for (int gc = g0; gc < g1; gc += TILES) {
-				acc += gemv_chunk<TILES, X_F32, DUMP_NONE>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false);
+				acc += gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false, nullptr, nullptr, 0,
+					norm);
 				__builtin_amdgcn_wave_barrier();
 			}
 		}
@@ -191,12 +202,15 @@ __global__ void ffn_empty_kernel(float* __restrict__ y, const float* __restrict_
 }
 
 template<int TILES, bool LOOP> static hipError_t launch_ffn_t(const ffn_args& a, unsigned grid, hipStream_t s) {
-	return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
+	if (a.norm_w) {
+		return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP, true>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
+	}
+	return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP, false>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
 }
 
 // n_ff % 128 == 0, K % 128 == 0, n_ff <= FFN_MAX_HIDDEN (checked by the caller).
-hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* residual, float* y, int64_t n_ff, int64_t K, int64_t n_out,
-	hipStream_t s) {
+hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* norm_w, float norm_eps, const float* residual, float* y, int64_t n_ff,
+	int64_t K, int64_t n_out, hipStream_t s) {
 	if (n_out == 0) {
 		return hipSuccess;
 	}
@@ -222,6 +236,8 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	a.w_up		 = static_cast<const uint8_t*>(w_up);
 	a.w_down	 = static_cast<const uint8_t*>(w_down);
 	a.x			 = x;
+	a.norm_w	 = norm_w;
+	a.norm_eps	 = norm_eps;
 	a.residual	 = residual;
 	a.y			 = y;
 	a.gate_up	 = sc.gate_up;

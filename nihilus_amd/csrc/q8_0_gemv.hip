@@ -115,10 +115,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* 
 //     depend on arrival order;
 //   * up to three weight matrices that share K and the activation row (q/k/v, gate/up) run as one launch:
 //     a bigger launch amortises the ramp-up and the tail.
-template<int TILES, bool XF32, int DUMP, bool LOOP>
+template<int TILES, bool XF32, int DUMP, bool LOOP, bool NORM>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, float* __restrict__ partials,
-	unsigned* __restrict__ counters, int groups, int split_shift, int groups_per_slot, int groups_rem) {
+	unsigned* __restrict__ counters, int groups, int split_shift, int groups_per_slot, int groups_rem, const float* __restrict__ norm_w, float norm_eps) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K]; // each wave's activation quants, block jj at 32*jj
+	__shared__ float norm_red[16];
+	__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1]; // each wave's slice of the norm weights
 	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
 	__shared__ float red[GEMV_WAVES][64];
 	__shared__ int last_flag;
@@ -139,13 +141,19 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	const uint8_t* w_strip = DUMP == DUMP_X ? nullptr : seg.W[sidx] + macro_offset(strip, 0, groups);
 	const int row_l		   = strip * STRIP_ROWS + (lane & 31);
 	float acc			   = 0.0f;
+	gemv_norm norm_state;
+	gemv_norm* norm = nullptr;
+	if constexpr (NORM) { // RMS norm * weight in front of the quantizer; an unsplit, single-chunk launch takes the sum from its slices
+		gemv_norm_begin(norm_state, static_cast<const float*>(xin), norm_w, xs_w[NORM ? wave : 0], norm_red, norm_eps, groups * GROUP_K, lane, wave, !LOOP && splits == 1);
+		norm = &norm_state;
+	}
 	if constexpr (!LOOP) {
 		// the host picked splits so that g1 - g0 <= TILES: straight-line code, every load of the wave in flight at once
-		acc = gemv_chunk<TILES, XF32, DUMP>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0);
+		acc = gemv_chunk<TILES, XF32, DUMP, NORM>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm);
 	} else {
 		// K too long for that within the host's scratch limits: walk the range in chunks of TILES groups
 		for (int gc = g0; gc < g1; gc += TILES) {
-			acc += gemv_chunk<TILES, XF32, DUMP>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0);
+			acc += gemv_chunk<TILES, XF32, DUMP, NORM>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm);
 			__builtin_amdgcn_wave_barrier(); // the next chunk overwrites this wave's LDS slice
 		}
 	}
@@ -255,7 +263,7 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	return hipSuccess;
 }
 
-template<int TILES, bool XF32, bool LOOP> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, hipStream_t s) {
+template<int TILES, bool XF32, bool LOOP, bool NORM> static hipError_t launch_gemv_tiled_n(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
 	const dim3 grid(static_cast<unsigned>(p.strips * p.splits)), block(GEMV_WAVES * 64);
 	int shift = 0;
 	while ((1 << shift) < p.splits) {
@@ -263,17 +271,27 @@ template<int TILES, bool XF32, bool LOOP> static hipError_t launch_gemv_tiled_t(
 	}
 	const int slots = p.splits * GEMV_WAVES, per_slot = p.groups / slots, rem = p.groups % slots;
 	if (dump_mode == DUMP_SUMS) {
-		gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem);
+		gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 		return hipGetLastError();
 	}
 	if (dump_mode == DUMP_X) {
-		gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem);
+		gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP>, grid, block, 0, s, seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem);
+	return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 }
 
-static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, void* dump, int dump_mode, hipStream_t s) {
+template<int TILES, bool XF32, bool LOOP> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
+	if constexpr (XF32) {
+		if (norm_w) {
+			return launch_gemv_tiled_n<TILES, XF32, LOOP, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
+		}
+	}
+	return launch_gemv_tiled_n<TILES, XF32, LOOP, false>(p, seg, x, dump, dump_mode, sc, nullptr, 0.0f, s);
+}
+
+static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, void* dump, int dump_mode, hipStream_t s,
+	const float* norm_w = nullptr, float norm_eps = 0.0f) {
 	gemv_segments seg{};
 	int64_t strips = 0;
 	for (int i = 0; i < GEMV_MAX_SEGMENTS; ++i) {
@@ -297,26 +315,26 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 		}
 	}
 	if (p.tiles > 4) { // K too long to keep every load in flight within the scratch limits: chunked walk
-		return x_is_f32 ? launch_gemv_tiled_t<4, true, true>(p, seg, x, dump, dump_mode, sc, s) : launch_gemv_tiled_t<4, false, true>(p, seg, x, dump, dump_mode, sc, s);
+		return x_is_f32 ? launch_gemv_tiled_t<4, true, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s) : launch_gemv_tiled_t<4, false, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 	}
 	const int tiles = p.tiles <= 1 ? 1 : (p.tiles <= 2 ? 2 : 4);
 	if (x_is_f32) {
 		switch (tiles) {
 			case 1:
-				return launch_gemv_tiled_t<1, true, false>(p, seg, x, dump, dump_mode, sc, s);
+				return launch_gemv_tiled_t<1, true, false>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 			case 2:
-				return launch_gemv_tiled_t<2, true, false>(p, seg, x, dump, dump_mode, sc, s);
+				return launch_gemv_tiled_t<2, true, false>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 			default:
-				return launch_gemv_tiled_t<4, true, false>(p, seg, x, dump, dump_mode, sc, s);
+				return launch_gemv_tiled_t<4, true, false>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 		}
 	}
 	switch (tiles) {
 		case 1:
-			return launch_gemv_tiled_t<1, false, false>(p, seg, x, dump, dump_mode, sc, s);
+			return launch_gemv_tiled_t<1, false, false>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 		case 2:
-			return launch_gemv_tiled_t<2, false, false>(p, seg, x, dump, dump_mode, sc, s);
+			return launch_gemv_tiled_t<2, false, false>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 		default:
-			return launch_gemv_tiled_t<4, false, false>(p, seg, x, dump, dump_mode, sc, s);
+			return launch_gemv_tiled_t<4, false, false>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 	}
 }
 
@@ -356,7 +374,7 @@ hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* 
 	return launch_gemv_blocks_t<4>(w, x, y, sums, static_cast<int>(N), static_cast<int>(K), s);
 }
 
-hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s) {
+hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s, const float* norm_w, float norm_eps) {
 	if (K == 0) {
 		for (int i = 0; i < count; ++i) {
 			if (N[i] > 0) {
@@ -365,13 +383,13 @@ hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const 
 		}
 		return hipGetLastError();
 	}
-	return launch_gemv_tiled_any(W, y, N, count, x, x_is_f32, K, nullptr, DUMP_NONE, s);
+	return launch_gemv_tiled_any(W, y, N, count, x, x_is_f32, K, nullptr, DUMP_NONE, s, x_is_f32 ? norm_w : nullptr, norm_eps);
 }
 
-hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s) {
+hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w, float norm_eps) {
 	const void* wl[1] = { nullptr }; // the dump variant never touches the weights
 	const int64_t n	  = STRIP_ROWS;
-	return launch_gemv_tiled_any(wl, nullptr, &n, 1, x, true, K, xq_blocks_out, DUMP_X, s);
+	return launch_gemv_tiled_any(wl, nullptr, &n, 1, x, true, K, xq_blocks_out, DUMP_X, s, norm_w, norm_eps);
 }
 
 } // namespace nh

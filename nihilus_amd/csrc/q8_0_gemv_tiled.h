@@ -29,9 +29,49 @@ enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
 enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2 };
 constexpr int FLAG_SPIN_LIMIT = 1 << 20;
 
-template<int TILES, int XMODE, int DUMP>
-__device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
-	int groups, int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2 = nullptr, const unsigned* __restrict__ flags = nullptr, unsigned epoch = 0) {
+// RMS norm * weight in front of the quantizer (X_F32 only).  The row's scale needs every element.  The fixed order
+// of the sum of squares (rms_run_* in q8_0_device.h) cuts the row into 16 runs exactly as an unsplit launch cuts K over
+// its 16 waves, so in that case the wave's activation slice, which it loads anyway, IS its share of the sum: no extra
+// load, one workgroup barrier while the weights are in flight (`from_slice`).  When K is split over workgroups or
+// walked in several chunks the slices do not cover the row, and the kernel works the scale out first from the row
+// itself (`ready`).  Loads return in issue order, so what the staging needs (the slice and its norm weights) is
+// requested BEFORE the weight stream: a load issued after it would only come back behind it.  The norm weights go
+// from memory straight into LDS (no destination registers: the kernel stays at two workgroups per CU).
+struct gemv_norm {
+	const float* w; // norm weight, fp32 [K]
+	float4* xs_w; // this wave's LDS slice for the norm weights of its activation slice (TILES * 32 float4)
+	float* red; // 16 floats of LDS
+	float eps;
+	float scale;
+	int K;
+	int wave;
+	bool ready; // scale holds the row's 1 / rms
+};
+__device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, const float* w, float4* xs_w, float* red, float eps, int K, int lane, int wave, bool from_slice) {
+	n.w		= w;
+	n.xs_w	= xs_w;
+	n.red	= red;
+	n.eps	= eps;
+	n.K		= K;
+	n.wave	= wave;
+	n.scale = 0.0f;
+	n.ready = false;
+	if (!from_slice) {
+		n.scale = rms_scale_workgroup(rms_run_sumsq(x, K / GROUP_K, wave, lane), red, wave, lane, K, eps);
+		n.ready = true;
+	}
+}
+
+//
+// CNT, the number of groups, is a template parameter although only the wave knows it at run time (gemv_chunk below
+// switches on it): loads complete in issue order and a wait names how many later ones may still be outstanding, so
+// the compiler can wait for the activation slice alone, with the weight loads still in flight, only where it can
+// count the weight loads.  With a run-time count it has to wait for everything, and the quantizer runs after the last
+// weight byte has landed instead of under the stream.
+template<int TILES, int XMODE, int DUMP, bool NORM, int CNT>
+__device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int groups,
+	int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2, const unsigned* __restrict__ flags, unsigned epoch, gemv_norm* norm) {
+	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
 	const int r	   = lane & 31;
 	const int half = lane >> 5;
@@ -42,6 +82,19 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 	uint32_t xr[XQ_LOADS];
 	float4 xf[XF_LOADS];
 	if constexpr (XMODE == X_F32) {
+		if constexpr (NORM) {
+			// memory -> LDS, no destination registers; issued before the slice loads, which the quantizer waits for:
+			// loads complete in issue order, so once the slice is there these are too
+			const float4* w4 = reinterpret_cast<const float4*>(norm->w + static_cast<int64_t>(gc) * GROUP_K);
+#pragma unroll
+			for (int i = 0; i < XF_LOADS; ++i) {
+				const int v = lane + 64 * i;
+				if (v < cnt * 32) { // 16 bytes per lane, lane l of the wave lands at xs_w[64 * i + l]
+					load_global_to_lds_b128(w4 + v, norm->xs_w + 64 * i);
+				}
+			}
+			asm volatile("" ::: "memory"); // the slice loads below are issued after these
+		}
 		const float4* x4 = reinterpret_cast<const float4*>(static_cast<const float*>(xin) + static_cast<int64_t>(gc) * GROUP_K);
 #pragma unroll
 		for (int i = 0; i < XF_LOADS; ++i) {
@@ -118,6 +171,27 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 
 	// ---- 3. stage the activation slice in LDS: quants 16-byte aligned per half block, scales as fp32 ----
 	if constexpr (XF32) {
+		if constexpr (NORM) {
+			if (!norm->ready) { // the slice is this wave's run of the row: reduce over the workgroup (one barrier, weights in flight)
+				float p = 0.0f;
+#pragma unroll
+				for (int i = 0; i < XF_LOADS; ++i) {
+					p = sumsq_fold(p, xf[i]); // lanes past the slice hold zeros, which leave p unchanged
+				}
+				norm->scale = rms_scale_workgroup(p, norm->red, norm->wave, lane, norm->K, norm->eps);
+				norm->ready = true;
+			}
+			// a use of the last slice register: the compiler has to wait for the slice here, which (issue order) covers the
+			// memory -> LDS loads; the LDS reads below may not move above this point
+			asm volatile("" ::"v"(xf[XF_LOADS - 1].w) : "memory");
+#pragma unroll
+			for (int i = 0; i < XF_LOADS; ++i) {
+				const int v = lane + 64 * i;
+				if (v < cnt * 32) {
+					xf[i] = norm_mul4(xf[i], norm->scale, norm->xs_w[v]);
+				}
+			}
+		}
 #pragma unroll
 		for (int i = 0; i < XF_LOADS; ++i) {
 			const int v = lane + 64 * i;
@@ -197,6 +271,28 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 		}
 	}
 	return acc;
+}
+
+template<int TILES, int XMODE, int DUMP, bool NORM = false>
+__device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
+	int groups, int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2 = nullptr, const unsigned* __restrict__ flags = nullptr, unsigned epoch = 0,
+	gemv_norm* norm = nullptr) {
+#define NH_CHUNK_CASE(C)                                                                                                                                              \
+	case C:                                                                                                                                                           \
+		if constexpr (C <= TILES) {                                                                                                                                   \
+			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0)>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm); \
+		}                                                                                                                                                             \
+		break;
+	switch (cnt) { // wave-uniform
+		NH_CHUNK_CASE(1)
+		NH_CHUNK_CASE(2)
+		NH_CHUNK_CASE(3)
+		NH_CHUNK_CASE(4)
+		default:
+			break;
+	}
+#undef NH_CHUNK_CASE
+	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm); // an idle wave (still takes part in barriers)
 }
 
 // Scratch of the K-split path (partial sums and arrival counters) and of the fused FFN launch (the gate and up

@@ -61,6 +61,69 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
 	}
 }
 
+// RMS norm * weight fused into the quantizer (the prologue of the q/k/v, gate/up and output projections in prefill):
+// one 1024-thread workgroup per row; the row's scale first (fixed-order sum of squares, see rms_scale_workgroup), then
+// every thread normalises and quantizes its float4s.  The row is read twice, the second time from cache.
+template<bool TILED>
+__global__ __launch_bounds__(1024) void rms_norm_quantize_kernel(const float* __restrict__ x, const float* __restrict__ norm_w, float eps, uint8_t* __restrict__ out, int64_t M, int K) {
+	__shared__ float red[16];
+	const int tid	  = threadIdx.x;
+	const int lane	  = tid & 63;
+	const int wave	  = tid >> 6;
+	const int64_t m	  = blockIdx.x; // row of the output, padding rows of a tiled output included
+	const int n4	  = K / 4;
+	const bool real	  = m < M;
+	const float4* x4  = reinterpret_cast<const float4*>(x + (real ? m : 0) * K);
+	const float4* w4  = reinterpret_cast<const float4*>(norm_w);
+	const float p = real ? rms_run_sumsq(x + m * K, K / GROUP_K, wave, lane) : 0.0f;
+	const float scale = rms_scale_workgroup(p, red, wave, lane, K, eps);
+	const int nb	  = K / QK;
+	for (int j0 = 0; j0 < n4; j0 += 1024) { // uniform trip count: whole 8-lane groups stay together in the quantizer
+		const int j = j0 + tid;
+		float4 v	= make_float4(0.f, 0.f, 0.f, 0.f);
+		if (real && j < n4) {
+			v = norm_mul4(x4[j], scale, w4[j]);
+		}
+		uint16_t dh;
+		const uint32_t packed = quantize_block_lane(v, &dh);
+		if (j >= n4) {
+			continue;
+		}
+		const int b	 = j >> 3;
+		const int jj = j & 7;
+		if constexpr (TILED) {
+			const int64_t strip = m / STRIP_ROWS;
+			const int r			= static_cast<int>(m % STRIP_ROWS);
+			uint8_t* macro		= out + macro_offset(strip, b / GROUP_BLOCKS, K / GROUP_K);
+			const int tq		= b % GROUP_BLOCKS;
+			const int l			= r + 32 * (jj >> 2);
+			*reinterpret_cast<uint32_t*>(macro + tq * TILE_BYTES + 16 * l + 4 * (jj & 3)) = packed;
+			if (jj == 0) {
+				*reinterpret_cast<uint16_t*>(macro + MACRO_D_OFFSET + 8 * r + 2 * tq) = dh;
+			}
+		} else {
+			uint8_t* o										 = out + (m * nb + b) * BLOCK_BYTES;
+			*reinterpret_cast<uint16_t*>(o + 2 + 4 * jj)	 = static_cast<uint16_t>(packed & 0xFFFFu);
+			*reinterpret_cast<uint16_t*>(o + 2 + 4 * jj + 2) = static_cast<uint16_t>(packed >> 16);
+			if (jj == 0) {
+				*reinterpret_cast<uint16_t*>(o) = dh;
+			}
+		}
+	}
+}
+
+hipError_t launch_rms_norm_quantize(const float* x, const float* norm_w, float eps, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s) {
+	const int64_t rows_out = tiled ? (M + STRIP_ROWS - 1) / STRIP_ROWS * STRIP_ROWS : M;
+	if (rows_out == 0 || K == 0) {
+		return hipSuccess;
+	}
+	const dim3 g(static_cast<unsigned>(rows_out)), b(1024);
+	if (tiled) {
+		return launch_kernel(KIND_QUANTIZE, rms_norm_quantize_kernel<true>, g, b, 0, s, x, norm_w, eps, static_cast<uint8_t*>(out), M, static_cast<int>(K));
+	}
+	return launch_kernel(KIND_QUANTIZE, rms_norm_quantize_kernel<false>, g, b, 0, s, x, norm_w, eps, static_cast<uint8_t*>(out), M, static_cast<int>(K));
+}
+
 template<bool SILU_MUL> static hipError_t launch_quantize_t(const float* x, const float* u, void* out, int64_t M, int64_t K, bool tiled, hipStream_t s) {
 	const int64_t rows_out = tiled ? (M + STRIP_ROWS - 1) / STRIP_ROWS * STRIP_ROWS : M;
 	const int64_t threads  = rows_out * (K / QK) * 8;

@@ -101,8 +101,10 @@ def get_rows(w: torch.Tensor, ids: torch.Tensor, n_rows: int, k: int, tiled: boo
     return (out, int(bad.item())) if count_invalid else out
 
 
-def ffn(w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, x: torch.Tensor, n_ff: int, k: int, n_out: int, residual: torch.Tensor | None = None) -> torch.Tensor:
-    """Decode-time FFN in one launch: W_down . Q(silu(W_gate . Q(x)) * (W_up . Q(x))) (+ residual); weights tiled, x fp32 [k]."""
+def ffn(w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, x: torch.Tensor, n_ff: int, k: int, n_out: int, residual: torch.Tensor | None = None,
+        norm_weight: torch.Tensor | None = None, eps: float = 0.0) -> torch.Tensor:
+    """Decode-time FFN in one launch: W_down . Q(silu(W_gate . Q(n)) * (W_up . Q(n))) (+ residual), n = x or its RMS norm
+    times norm_weight; weights tiled, x fp32 [k]."""
     w_gate, w_up, w_down = _dev(w_gate, torch.uint8, "w_gate"), _dev(w_up, torch.uint8, "w_up"), _dev(w_down, torch.uint8, "w_down")
     x = _dev(x, torch.float32, "x")
     if w_gate.numel() != tiled_bytes(n_ff, k) or w_up.numel() != tiled_bytes(n_ff, k) or w_down.numel() != tiled_bytes(n_out, n_ff) or x.numel() != k:
@@ -111,8 +113,11 @@ def ffn(w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, x: torch
         residual = _dev(residual, torch.float32, "residual")
         if residual.numel() != n_out:
             raise ValueError("residual must hold n_out values")
+    if norm_weight is not None and _dev(norm_weight, torch.float32, "norm_weight").numel() != k:
+        raise ValueError("norm_weight must hold k floats")
     y = torch.empty(n_out, dtype=torch.float32, device=x.device)
     _lib.check("nh_q8_0_ffn_f32", _lib.lib().nh_q8_0_ffn_f32(w_gate.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), x.data_ptr(),
+                                                           norm_weight.data_ptr() if norm_weight is not None else None, eps,
                                                            residual.data_ptr() if residual is not None else None, y.data_ptr(), n_ff, k, n_out, _stream()))
     return y
 
@@ -135,8 +140,10 @@ def gemv(w: torch.Tensor, xq_blocks: torch.Tensor, n: int, k: int, tiled: bool) 
     return y
 
 
-def gemv_f32(w_tiled: list[torch.Tensor] | torch.Tensor, x: torch.Tensor, n: list[int] | int, k: int) -> list[torch.Tensor] | torch.Tensor:
-    """Fused quantize + mat-vec on tiled weights; a list of up to 3 weights sharing x and k runs as one launch."""
+def gemv_f32(w_tiled: list[torch.Tensor] | torch.Tensor, x: torch.Tensor, n: list[int] | int, k: int, norm_weight: torch.Tensor | None = None,
+             eps: float = 0.0) -> list[torch.Tensor] | torch.Tensor:
+    """Fused quantize + mat-vec on tiled weights; a list of up to 3 weights sharing x and k runs as one launch.
+    With norm_weight the activation is RMS-normalised and multiplied by it first, inside the same launch."""
     import ctypes as C
 
     single = not isinstance(w_tiled, (list, tuple))
@@ -153,16 +160,42 @@ def gemv_f32(w_tiled: list[torch.Tensor] | torch.Tensor, x: torch.Tensor, n: lis
     wp = (C.c_void_p * cnt)(*[w.data_ptr() for w in ws])
     yp = (C.c_void_p * cnt)(*[y.data_ptr() for y in ys])
     np_ = (C.c_int64 * cnt)(*ns)
-    _lib.check("nh_q8_0_gemv_tiled_multi_f32", _lib.lib().nh_q8_0_gemv_tiled_multi_f32(wp, yp, np_, cnt, x.data_ptr(), k, _stream()))
+    if norm_weight is not None:
+        nw = _dev(norm_weight, torch.float32, "norm_weight")
+        if nw.numel() != k:
+            raise ValueError("norm_weight must hold k floats")
+        _lib.check("nh_q8_0_gemv_tiled_multi_norm_f32", _lib.lib().nh_q8_0_gemv_tiled_multi_norm_f32(wp, yp, np_, cnt, x.data_ptr(), nw.data_ptr(), eps, k, _stream()))
+    else:
+        _lib.check("nh_q8_0_gemv_tiled_multi_f32", _lib.lib().nh_q8_0_gemv_tiled_multi_f32(wp, yp, np_, cnt, x.data_ptr(), k, _stream()))
     return ys[0] if single else ys
 
 
-def debug_fused_quantize(x: torch.Tensor) -> torch.Tensor:
-    """The activation row exactly as the fused mat-vec stages it, as packed blocks."""
+def debug_fused_quantize(x: torch.Tensor, norm_weight: torch.Tensor | None = None, eps: float = 0.0) -> torch.Tensor:
+    """The activation row exactly as the fused mat-vec stages it (after the RMS norm, if a norm weight is given), as packed blocks."""
     x = _dev(x, torch.float32, "x")
     k = x.numel()
     out = torch.zeros(blocks_bytes(1, k), dtype=torch.uint8, device=x.device)
-    _lib.check("nh_q8_0_debug_fused_quantize", _lib.lib().nh_q8_0_debug_fused_quantize(x.data_ptr(), out.data_ptr(), k, _stream()))
+    if norm_weight is not None:
+        nw = _dev(norm_weight, torch.float32, "norm_weight")
+        _lib.check("nh_q8_0_debug_fused_norm_quantize", _lib.lib().nh_q8_0_debug_fused_norm_quantize(x.data_ptr(), nw.data_ptr(), eps, out.data_ptr(), k, _stream()))
+    else:
+        _lib.check("nh_q8_0_debug_fused_quantize", _lib.lib().nh_q8_0_debug_fused_quantize(x.data_ptr(), out.data_ptr(), k, _stream()))
+    return out
+
+
+def rms_norm_quantize(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, tiled: bool = False) -> torch.Tensor:
+    """quantize_row_q8_0((x * 1/rms(x)) * norm_weight) for fp32 [M, K] (or [K]) rows, one kernel; output as quantize_row_q8_0."""
+    x, nw = _dev(x, torch.float32, "x"), _dev(norm_weight, torch.float32, "norm_weight")
+    x2 = x.reshape(1, -1) if x.dim() == 1 else x
+    m, k = x2.shape
+    if nw.numel() != k:
+        raise ValueError("norm_weight must hold k floats")
+    if tiled:
+        out = torch.empty(tiled_bytes(m, k), dtype=torch.uint8, device=x.device)
+        _lib.check("nh_q8_0_rms_norm_quantize_tiled", _lib.lib().nh_q8_0_rms_norm_quantize_tiled(x2.data_ptr(), nw.data_ptr(), eps, out.data_ptr(), m, k, _stream()))
+        return out
+    out = torch.empty((m, blocks_bytes(1, k)), dtype=torch.uint8, device=x.device)
+    _lib.check("nh_q8_0_rms_norm_quantize", _lib.lib().nh_q8_0_rms_norm_quantize(x2.data_ptr(), nw.data_ptr(), eps, out.data_ptr(), m, k, _stream()))
     return out
 
 

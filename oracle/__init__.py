@@ -52,6 +52,9 @@ _a_fp32_to_fp16 = _sig(_a, "nha_fp32_to_fp16", C.c_uint16, C.c_float)
 _q8_bytes = _sig(_o, "nho_q8_0_bytes", _i64, _i64, _i64)
 _dequant = _sig(_o, "nho_dequantize_row_q8_0", None, _vp, _vp, _i64)
 _get_rows = _sig(_o, "nho_get_rows_q8_0", _i64, _vp, _vp, _vp, _i64, _i64, _i64)
+_rms_scale = _sig(_o, "nho_rms_norm_scale", C.c_float, _vp, _i64, C.c_float)
+_rms_mul_row = _sig(_o, "nho_rms_norm_mul_row", None, _vp, _vp, C.c_float, _vp, _i64)
+_rms_quant_rows = _sig(_o, "nho_rms_norm_quantize_rows_q8_0", None, _vp, _vp, C.c_float, _vp, _i64, _i64, _vp)
 _expf = _sig(_o, "nho_expf", C.c_float, C.c_float)
 _silu_mul = _sig(_o, "nho_silu_mul", C.c_float, C.c_float, C.c_float)
 _silu_mul_quant_rows = _sig(_o, "nho_silu_mul_quantize_rows_q8_0", None, _vp, _vp, _vp, _i64, _i64)
@@ -144,6 +147,31 @@ def get_rows(blocks: np.ndarray, ids: np.ndarray, n_rows: int, k: int):
     out = np.empty((ids.size, k), dtype=np.float32)
     bad = _get_rows(_ptr(b), _ptr(ids), _ptr(out), ids.size, n_rows, k)
     return out, int(bad)
+
+
+def rms_norm_scale(x: np.ndarray, eps: float) -> float:
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    return float(_rms_scale(_ptr(x), x.size, eps))
+
+
+def rms_norm_mul(x: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
+    """(x * 1/rms(x)) * w for one fp32 row, in the checker's fixed order."""
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    w = np.ascontiguousarray(w, dtype=np.float32).ravel()
+    y = np.empty_like(x)
+    _rms_mul_row(_ptr(x), _ptr(w), eps, _ptr(y), x.size)
+    return y
+
+
+def rms_norm_quantize_rows(x: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
+    """x: fp32 [m, k], w: fp32 [k]; returns uint8 [m, (k//32)*34] = quantize_rows(rms_norm(x) * w)."""
+    x = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32).ravel()
+    m, k = x.shape
+    out = np.empty((m, k // QK * BLOCK_BYTES), dtype=np.uint8)
+    tmp = np.empty(k, dtype=np.float32)
+    _rms_quant_rows(_ptr(x), _ptr(w), eps, _ptr(out), m, k, _ptr(tmp))
+    return out
 
 
 def expf(x: np.ndarray) -> np.ndarray:

@@ -27,6 +27,10 @@
  *                                        decodes to the constant r (index order), out-of-range ids.  The
  *                                        reference's dump of this op's output (inp_embd) covers a vocabulary row
  *                                        whose bytes are not in the dumps, so it cannot be replayed end to end.
+ *   nho_rms_norm_*                       the reference's rms_norm has no live body and an ISA-dependent sqrtf_fast:
+ *                                        pinned against float64 (sum of squares, scale, normalised row), by exact
+ *                                        invariance under scaling the row by powers of two (eps = 0), and by
+ *                                        constant rows whose answer is known in closed form.
  *   nho_expf / nho_silu_mul              no reference body exists (its silu kernels are empty): pinned against the
  *                                        correctly rounded double-precision value, <= 2 ulp over a dense sweep of
  *                                        the whole clamped range plus the special points; silu against float64.
@@ -180,6 +184,71 @@ int64_t nho_get_rows_q8_0(const void* vw, const int32_t* ids, float* out, int64_
 		nho_dequantize_row_q8_0(w + id * row_size, out + t * k, k);
 	}
 	return invalid;
+}
+
+/* ---------------------------------------------------------------- RMS norm */
+
+/* 1 / sqrt(mean(x^2) + eps) with the sum of squares taken in the order of the GPU kernels' 1024-thread workgroup:
+ * the row's G = k / 128 groups are cut into 16 contiguous runs (q = G / 16 groups each, the first G % 16 runs one more);
+ * lane l of wave w folds the float4s l, l + 64, ... of run w by fma; each 64-lane wave is reduced by an xor butterfly
+ * over lane distances 32, 16, ..., 1; the 16 wave sums are added in wave order.  The rms_norm node of the reference's
+ * graph (infra/core_traits.hpp:570, :971, :1186); its dead CPU attempt (cpu/avx_2.hpp:5331-5347) sums 8 AVX lanes and
+ * calls sqrtf_fast, which is vsqrt on NEON and a bit trick elsewhere (cpu/common.hpp:310, :448): here the square root
+ * and the divides are the IEEE ones.  k % 128 == 0. */
+float nho_rms_norm_scale(const float* x, int64_t k, float eps) {
+	float wave_sum[16];
+	const int64_t groups = k / 128, q = groups / 16, r = groups % 16;
+	for (int w = 0; w < 16; ++w) {
+		const int64_t g0 = w * q + (w < r ? w : r);
+		const int64_t n4 = (q + (w < r ? 1 : 0)) * 32;
+		const float* run = x + g0 * 128;
+		float lane[64], next[64];
+		for (int l = 0; l < 64; ++l) {
+			float p = 0.0f;
+			for (int64_t j = l; j < n4; j += 64) {
+				for (int e = 0; e < 4; ++e) {
+					p = fmaf(run[4 * j + e], run[4 * j + e], p);
+				}
+			}
+			lane[l] = p;
+		}
+		for (int off = 32; off >= 1; off >>= 1) {
+			for (int l = 0; l < 64; ++l) {
+				volatile float s = lane[l] + lane[l ^ off];
+				next[l]			 = s;
+			}
+			memcpy(lane, next, sizeof(lane));
+		}
+		wave_sum[w] = lane[0];
+	}
+	volatile float sum = wave_sum[0];
+	for (int w = 1; w < 16; ++w) {
+		sum = sum + wave_sum[w];
+	}
+	volatile float mean = sum / (float)k;
+	volatile float arg	= mean + eps;
+	volatile float root = sqrtf(arg);
+	return 1.0f / root;
+}
+
+/* y_i = (x_i * scale) * w_i: the rms_norm node, then the mul node with the norm weight (infra/core_traits.hpp:570-573) */
+void nho_rms_norm_mul_row(const float* x, const float* w, float eps, float* y, int64_t k) {
+	const float scale = nho_rms_norm_scale(x, k, eps);
+	for (int64_t i = 0; i < k; ++i) {
+		volatile float t = x[i] * scale;
+		y[i]			 = t * w[i];
+	}
+}
+
+void nho_quantize_row_q8_0(const float* x, void* vy, int64_t k);
+
+/* xq[m] = quantize_row_q8_0(rms_norm(x[m]) * w), m rows of k */
+void nho_rms_norm_quantize_rows_q8_0(const float* x, const float* w, float eps, void* vy, int64_t m, int64_t k, float* scratch_row) {
+	uint8_t* y = (uint8_t*)vy;
+	for (int64_t r = 0; r < m; ++r) {
+		nho_rms_norm_mul_row(x + r * k, w, eps, scratch_row, k);
+		nho_quantize_row_q8_0(scratch_row, y + r * (k / NHO_QK) * NHO_BLOCK_BYTES, k);
+	}
 }
 
 /* ---------------------------------------------------------------- FFN activation */

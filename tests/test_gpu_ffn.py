@@ -138,17 +138,17 @@ def test_ffn_empty_and_errors(q8):
     r = torch.arange(32, dtype=torch.float32, device="cuda")
     y = torch.full((32,), 7.0, dtype=torch.float32, device="cuda")
     p = lambda t: t.data_ptr()
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, p(y), 128, 128, 0, None) == 0
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), p(r), p(y), 0, 128, 32, None) == 0  # empty hidden dim: y = residual
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, None, p(y), 128, 128, 0, None) == 0
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, p(r), p(y), 0, 128, 32, None) == 0  # empty hidden dim: y = residual
     assert torch.equal(y, r)
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, p(y), 128, 0, 32, None) == 0
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, None, p(y), 128, 0, 32, None) == 0
     assert torch.equal(y, torch.zeros_like(y))
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, p(y), 96, 128, 32, None) == -3
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, p(y), 128, 96, 32, None) == -3
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, p(y), 65536 + 128, 128, 32, None) == -5
-    assert lib.nh_q8_0_ffn_f32(None, p(w), p(w), p(x), None, p(y), 128, 128, 32, None) == -1
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, None, 128, 128, 32, None) == -1
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x) + 4, None, p(y), 128, 128, 32, None) == -2
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, None, p(y), 96, 128, 32, None) == -3
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, None, p(y), 128, 96, 32, None) == -3
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, None, p(y), 65536 + 128, 128, 32, None) == -5
+    assert lib.nh_q8_0_ffn_f32(None, p(w), p(w), p(x), None, 0.0, None, p(y), 128, 128, 32, None) == -1
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, None, None, 128, 128, 32, None) == -1
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x) + 4, None, 0.0, None, p(y), 128, 128, 32, None) == -2
     # zero weights: g = u = 0, activation 0, y = residual exactly
-    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), p(r), p(y), 128, 128, 32, None) == 0
+    assert lib.nh_q8_0_ffn_f32(p(w), p(w), p(w), p(x), None, 0.0, p(r), p(y), 128, 128, 32, None) == 0
     assert torch.equal(y, r)

@@ -1,0 +1,88 @@
+"""GPU: RMS norm * weight fused into the quantizer (stand-alone kernel, inside the mat-vec, inside the one-launch FFN),
+byte-exact against the CPU checker, which takes the sum of squares in the same fixed order."""
+import numpy as np
+import pytest
+
+from helpers import REL_L2_TOL, random_blocks, rel_l2, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+EPS = 1e-5
+
+
+def row_inputs(seed, m, k, scale=3.0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((m, k)) * scale).astype(np.float32)
+    w = (1 + 0.2 * rng.standard_normal(k)).astype(np.float32)
+    return x, w
+
+
+@pytest.mark.parametrize("m,k", [(1, 128), (1, 4096), (5, 8192), (33, 1024), (3, 14336), (64, 4096)])
+def test_rms_norm_quantize_bit_exact(q8, oracle, m, k):
+    x, w = row_inputs(m + k, m, k)
+    want = oracle.rms_norm_quantize_rows(x, w, EPS)
+    assert np.array_equal(to_host(q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS)), want)
+    tiled = q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS, tiled=True)
+    assert np.array_equal(to_host(q8.untile(tiled, m, k)).reshape(m, -1), want)
+
+
+@pytest.mark.parametrize("k", [128, 1024, 4096, 8192, 14336])
+def test_norm_inside_the_mat_vec_stages_the_same_bytes(q8, oracle, k):
+    # K <= 8192: the in-chunk reduction (weights already in flight); 14336: the up-front form
+    x, w = row_inputs(k, 1, k, scale=0.5)
+    want = oracle.rms_norm_quantize_rows(x, w, EPS)[0]
+    assert np.array_equal(to_host(q8.debug_fused_quantize(to_dev(x[0]), to_dev(w), EPS)), want)
+    assert np.array_equal(to_host(q8.debug_fused_quantize(to_dev(x[0]))), oracle.quantize_rows(x)[0])  # and without a norm, as before
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (100, 1024), (1024, 8192), (64, 14336), (128256, 4096)])
+def test_norm_mat_vec_matches_two_step_form(q8, oracle, n, k):
+    x, w = row_inputs(n + k, 1, k)
+    wt = q8.tile(q8.fill_weight_blocks(n, n, k), n, k)
+    y = q8.gemv_f32(wt, to_dev(x[0]), n, k, norm_weight=to_dev(w), eps=EPS)
+    xq = q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS)
+    assert np.array_equal(to_host(y), to_host(q8.gemv(wt, xq.reshape(-1), n, k, True)))  # same quantized row, same mat-vec
+    if n <= 4096:
+        wb = oracle.fill_weights(n, n, k)
+        assert rel_l2(to_host(y), oracle.gemv(wb, oracle.rms_norm_quantize_rows(x, w, EPS)[0], n, k)) <= REL_L2_TOL
+
+
+def test_norm_qkv_as_one_launch(q8, oracle):
+    k, ns = 4096, [4096, 1024, 1024]
+    x, w = row_inputs(9, 1, k)
+    wts = [q8.tile(q8.fill_weight_blocks(20 + i, n, k), n, k) for i, n in enumerate(ns)]
+    ys = q8.gemv_f32(wts, to_dev(x[0]), ns, k, norm_weight=to_dev(w), eps=EPS)
+    xq = oracle.rms_norm_quantize_rows(x, w, EPS)[0]
+    for i, n in enumerate(ns):
+        assert rel_l2(to_host(ys[i]), oracle.gemv(oracle.fill_weights(20 + i, n, k), xq, n, k)) <= REL_L2_TOL
+
+
+def test_norm_inside_the_one_launch_ffn(q8, oracle):
+    n_ff, k, n_out = 2048, 1024, 512
+    rng = np.random.default_rng(4)
+    wg, wu, wd = random_blocks(rng, n_ff, k, 0.02), random_blocks(rng, n_ff, k, 0.02), random_blocks(rng, n_out, n_ff, 0.02)
+    x, w = row_inputs(5, 1, k)
+    t = [q8.tile(to_dev(b), r, c) for b, r, c in ((wg, n_ff, k), (wu, n_ff, k), (wd, n_out, n_ff))]
+    y = q8.ffn(t[0], t[1], t[2], to_dev(x[0]), n_ff, k, n_out, norm_weight=to_dev(w), eps=EPS)
+    g, u = q8.debug_ffn_gate_up(n_ff)
+    xq = oracle.rms_norm_quantize_rows(x, w, EPS)[0]
+    assert rel_l2(to_host(g), oracle.gemv(wg, xq, n_ff, k)) <= REL_L2_TOL and rel_l2(to_host(u), oracle.gemv(wu, xq, n_ff, k)) <= REL_L2_TOL
+    aq = oracle.silu_mul_quantize_rows(to_host(g), to_host(u))[0]
+    assert rel_l2(to_host(y), oracle.gemv(wd, aq, n_out, n_ff)) <= 2e-6
+
+
+def test_rms_norm_errors(q8):
+    import torch
+
+    from nihilus_amd import _lib
+
+    lib = _lib.lib()
+    x = torch.ones(128, dtype=torch.float32, device="cuda")
+    out = torch.zeros(4 * 34, dtype=torch.uint8, device="cuda")
+    p = lambda t: t.data_ptr()
+    assert lib.nh_q8_0_rms_norm_quantize(p(x), p(x), 1e-5, p(out), 1, 100, None) == -3
+    assert lib.nh_q8_0_rms_norm_quantize(p(x), None, 1e-5, p(out), 1, 128, None) == -1
+    assert lib.nh_q8_0_rms_norm_quantize(p(x), p(x), -1.0, p(out), 1, 128, None) == -6
+    assert lib.nh_q8_0_rms_norm_quantize(p(x), p(x) + 4, 1e-5, p(out), 1, 128, None) == -2
+    assert lib.nh_q8_0_rms_norm_quantize(p(x), p(x), 1e-5, p(out), 1, 96, None) == -3  # the sum order is defined on 128-value groups
+    assert lib.nh_q8_0_rms_norm_quantize(p(x), p(x), 1e-5, p(out), 0, 128, None) == 0
