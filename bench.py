@@ -30,9 +30,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 GATE_N, HIDDEN, FFN = 14336, 4096, 14336
 # HBM bytes per launch of the dominant kernel, mean over the step's two launches: FETCH_SIZE and WRITE_SIZE from two
 # rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for a plain 64 MiB copy
-# (FETCH_SIZE x 1.99928, WRITE_SIZE x 1.0).  A hardware-counter figure cannot be taken live; this is the recorded one.
+# (FETCH_SIZE x 1.99927, WRITE_SIZE x 1.0).  A hardware-counter figure cannot be taken live; this is the recorded one.
 # Keyed by --ffn-mode; None = not measured yet for that mode.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"batch": 93907580, "fused": None}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"batch": 93887437, "fused": 187808256}
 
 
 def weight_bytes(n: int, k: int) -> int:
