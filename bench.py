@@ -61,7 +61,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
     ap.add_argument("--calibration-copies", type=int, default=0, help="run this many plain 64 MiB device copies first (a known-size kernel to scale hardware byte counters by)")
-    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows"], default="ffn_decode",
+    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
     ap.add_argument("--ffn-mode", choices=["batch", "fused"], default="batch",
@@ -298,6 +298,38 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
             "roofline": {"bound": "hbm", "kernel": "nh::quantize_kernel<true>", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n},
         }
+
+    if kind == "crossover":
+        # M in {1, 8, 32, 128, 512} against the same two weights: where the mat-vec (HBM-bound) hands over to the
+        # weight-streaming MFMA kernel (M <= 64) and that to the MFMA tile kernel (compute-bound)
+        shapes = [(4096, K), (14336, K)]
+        ws = [q8_0.tile(q8_0.fill_weight_blocks(3 + i, n, k), n, k) for i, (n, k) in enumerate(shapes)]
+        rows = []
+        for m in (1, 8, 32, 64, 128, 512):
+            xm = x[:m].contiguous()
+            ws_bytes = max(256, lib.nh_q8_0_mul_mat_workspace_bytes(m, K))
+            wsp = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+            for w, (n, k) in zip(ws, shapes):
+                c = torch.empty((m, n), dtype=torch.float32, device=x.device)
+
+                def fn():
+                    _lib.check("nh_q8_0_mul_mat", lib.nh_q8_0_mul_mat(w.data_ptr(), xm.data_ptr(), c.data_ptr(), m, n, k, wsp.data_ptr(), ws_bytes, stream))
+
+                for _ in range(warmup):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    fn()
+                torch.cuda.synchronize()
+                sec = (time.perf_counter() - t0) / steps
+                wbytes = n * (k // 32) * 34
+                rows.append({"M": m, "N": n, "K": k, "us": round(sec * 1e6, 2), "weight_GBs": round(wbytes / sec / 1e9, 1), "TOPs": round(2.0 * m * n * k / sec / 1e12, 2),
+                             "pct_hbm": round(100 * wbytes / sec / 1e9 / HBM_PEAK_GBS, 1), "pct_mfma": round(100 * 2.0 * m * n * k / sec / 1e12 / INT8_MFMA_PEAK_TOPS, 2)})
+        return {"metric": "Q8_0 mul_mat (quantize + mat-vec / mat-mat) time against M", "unit": "us", "n_gpus": 1, "steps": steps, "warmup": warmup, "higher_is_better": False,
+                "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate", "data": "synthetic",
+                "config": {"workload": "nh_q8_0_mul_mat, fp32 activations [M x 4096] x Q8_0 W [4096x4096] and [14336x4096], activation quantize included, weights cache-resident "
+                           "(17.8 / 62.4 MB against a 256 MB last-level cache): the GEMV -> GEMM crossover, not an HBM figure"}, "rows": rows}
 
     if kind == "get_rows":
         n_rows = 128256  # LLaMA-3 vocabulary; token_embd.weight [4096 x 128256] Q8_0 = 558 MB, rows picked at random

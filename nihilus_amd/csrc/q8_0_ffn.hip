@@ -38,8 +38,7 @@ struct ffn_args {
 	float* act_d; // scratch: its scales
 	unsigned* flags; // scratch: one word per block
 	unsigned epoch;
-	float* partials;
-	unsigned* counters;
+	uint64_t* tagged; // scratch: tagged partial sums of the down projection's K split
 	int n_ff, n_out;
 	int groups_p, groups_c; // K / 128, n_ff / 128
 	int producers; // n_ff / 32
@@ -51,7 +50,6 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K];
 	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
 	__shared__ float red[GEMV_WAVES][64];
-	__shared__ int last_flag;
 
 	const int tid  = threadIdx.x;
 	const int lane = tid & 63;
@@ -158,38 +156,9 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 		}
 		return;
 	}
-	// K split over several workgroups: as in the plain mat-vec, the last to arrive adds the partial sums in split order
+	// K split over several workgroups: as in the plain mat-vec
 	if (tid < STRIP_ROWS) {
-		__hip_atomic_store(&a.partials[(static_cast<int64_t>(gstrip) * splits + split) * STRIP_ROWS + tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-	}
-	wait_stores_acknowledged();
-	__syncthreads();
-	if (tid == 0) {
-		const unsigned prev = __hip_atomic_fetch_add(&a.counters[gstrip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-		const int last		= (prev == static_cast<unsigned>(splits - 1));
-		if (last) {
-			__hip_atomic_store(&a.counters[gstrip], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-		}
-		last_flag = last;
-	}
-	__syncthreads();
-	if (last_flag && tid < STRIP_ROWS && row < a.n_out) {
-		const float* mine = a.partials + static_cast<int64_t>(gstrip) * splits * STRIP_ROWS + tid;
-		float sum		  = 0.0f;
-		for (int sp0 = 0; sp0 < splits; sp0 += 8) {
-			float v[8];
-#pragma unroll
-			for (int u = 0; u < 8; ++u) {
-				v[u] = (sp0 + u < splits) ? __hip_atomic_load(&mine[(sp0 + u) * STRIP_ROWS], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
-			}
-#pragma unroll
-			for (int u = 0; u < 8; ++u) {
-				if (sp0 + u < splits) {
-					sum += v[u];
-				}
-			}
-		}
-		a.y[row] = a.residual ? sum + a.residual[row] : sum;
+		split_k_finish(a.tagged, a.epoch, gstrip, splits, split, tid, total, a.y, row, a.n_out, a.residual);
 	}
 }
 
@@ -245,8 +214,7 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	a.act_d		 = sc.act_d;
 	a.flags		 = sc.flags;
 	a.epoch		 = sc.epoch;
-	a.partials	 = sc.partials;
-	a.counters	 = sc.counters;
+	a.tagged	 = sc.tagged;
 	a.n_ff		 = static_cast<int>(n_ff);
 	a.n_out		 = static_cast<int>(n_out);
 	a.groups_p	 = static_cast<int>(K / GROUP_K);

@@ -116,15 +116,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* 
 //   * up to three weight matrices that share K and the activation row (q/k/v, gate/up) run as one launch:
 //     a bigger launch amortises the ramp-up and the tail.
 template<int TILES, bool XF32, int DUMP, bool LOOP, bool NORM>
-__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, float* __restrict__ partials,
-	unsigned* __restrict__ counters, int groups, int split_shift, int groups_per_slot, int groups_rem, const float* __restrict__ norm_w, float norm_eps) {
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, uint64_t* __restrict__ tagged,
+	unsigned epoch, int groups, int split_shift, int groups_per_slot, int groups_rem, const float* __restrict__ norm_w, float norm_eps) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K]; // each wave's activation quants, block jj at 32*jj
 	__shared__ float norm_red[16];
 	__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1]; // each wave's slice of the norm weights
 	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
 	__shared__ float red[GEMV_WAVES][64];
-	__shared__ int last_flag;
-
 	const int tid	 = threadIdx.x;
 	const int lane	 = tid & 63;
 	const int wave	 = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform by construction: keep it (and all that follows from it) scalar
@@ -180,44 +178,9 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 		return;
 	}
 
-	// ---- K split over several workgroups: publish partial sums, the last arriver adds them in split order ----
-	// Each XCD has its own L2, so data that crosses workgroups goes through device-scope atomic stores and loads
-	// (written through to / read from the memory side).  A device-wide fence would also order them, but it writes
-	// back and invalidates the whole L2 under the other workgroups' streaming loads; waiting for the stores to be
-	// acknowledged before the arrival count is bumped is all the ordering this hand-off needs.
+	// ---- K split over several workgroups ----
 	if (tid < STRIP_ROWS) {
-		__hip_atomic_store(&partials[(static_cast<int64_t>(gstrip) * splits + split) * STRIP_ROWS + tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-	}
-	wait_stores_acknowledged();
-	__syncthreads();
-	if (tid == 0) {
-		const unsigned prev = __hip_atomic_fetch_add(&counters[gstrip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-		const int last		= (prev == static_cast<unsigned>(splits - 1));
-		if (last) {
-			__hip_atomic_store(&counters[gstrip], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // all arrived: ready for the next launch
-		}
-		last_flag = last;
-	}
-	__syncthreads();
-	if (last_flag && tid < STRIP_ROWS && row < N) {
-		// all partial sums requested before the first is waited for (they come from the memory side, ~1 us each if
-		// taken one at a time), then added in split order
-		const float* mine = partials + static_cast<int64_t>(gstrip) * splits * STRIP_ROWS + tid;
-		float sum		  = 0.0f;
-		for (int sp0 = 0; sp0 < splits; sp0 += 8) {
-			float v[8];
-#pragma unroll
-			for (int u = 0; u < 8; ++u) {
-				v[u] = (sp0 + u < splits) ? __hip_atomic_load(&mine[(sp0 + u) * STRIP_ROWS], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
-			}
-#pragma unroll
-			for (int u = 0; u < 8; ++u) {
-				if (sp0 + u < splits) {
-					sum += v[u];
-				}
-			}
-		}
-		y[row] = sum;
+		split_k_finish(tagged, epoch, gstrip, splits, split, tid, total, y, row, N, nullptr);
 	}
 }
 
@@ -234,21 +197,20 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	}
 	std::lock_guard<std::mutex> g(lock);
 	gemv_scratch& sc = per_device[dev];
-	if (!sc.partials) {
+	if (!sc.tagged) {
 		void* p			   = nullptr;
-		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 4 + GEMV_MAX_SPLIT_STRIPS * 4 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * (8 + 1 + 1) * 4;
+		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * (8 + 1 + 1) * 4;
 		e				   = hipMalloc(&p, bytes);
 		if (e != hipSuccess) {
 			return e;
 		}
-		e = hipMemset(p, 0, bytes); // synchronous, once: counters start at zero and every launch leaves them at zero; flags start at epoch 0
+		e = hipMemset(p, 0, bytes); // synchronous, once: every tag and flag starts at epoch 0, which no launch uses
 		if (e != hipSuccess) {
 			(void)hipFree(p);
 			return e;
 		}
-		sc.partials = static_cast<float*>(p);
-		sc.counters = reinterpret_cast<unsigned*>(sc.partials + static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS);
-		sc.gate_up	= reinterpret_cast<float*>(sc.counters + GEMV_MAX_SPLIT_STRIPS);
+		sc.tagged  = static_cast<uint64_t*>(p);
+		sc.gate_up = reinterpret_cast<float*>(sc.tagged + static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS);
 		sc.act_q	= reinterpret_cast<uint32_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
 		sc.act_d	= reinterpret_cast<float*>(sc.act_q + (FFN_MAX_HIDDEN / STRIP_ROWS) * 8);
 		sc.flags	= reinterpret_cast<unsigned*>(sc.act_d + FFN_MAX_HIDDEN / STRIP_ROWS);
@@ -271,14 +233,14 @@ template<int TILES, bool XF32, bool LOOP, bool NORM> static hipError_t launch_ge
 	}
 	const int slots = p.splits * GEMV_WAVES, per_slot = p.groups / slots, rem = p.groups % slots;
 	if (dump_mode == DUMP_SUMS) {
-		gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+		gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 		return hipGetLastError();
 	}
 	if (dump_mode == DUMP_X) {
-		gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+		gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.partials, sc.counters, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+	return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 }
 
 template<int TILES, bool XF32, bool LOOP> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
@@ -309,7 +271,7 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 	const gemv_plan p = plan_gemv(strips, K);
 	gemv_scratch sc;
 	if (p.splits > 1) {
-		const hipError_t e = get_gemv_scratch(&sc);
+		const hipError_t e = get_gemv_scratch(&sc, true);
 		if (e != hipSuccess) {
 			return e;
 		}

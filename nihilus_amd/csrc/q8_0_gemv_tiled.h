@@ -295,15 +295,50 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm); // an idle wave (still takes part in barriers)
 }
 
-// Scratch of the K-split path (partial sums and arrival counters) and of the fused FFN launch (the gate and up
+// K split over several workgroups: each publishes the 32 partial sums of its share, tagged with the launch's epoch
+// (one 64-bit device-scope store per row: tag and value can never be seen apart), waits for the acknowledgement, then
+// reads every share of its strip.  A row whose shares all carry the epoch is summed in split order and stored; the
+// workgroup whose store was performed last is certain to see them all, an earlier one may too and then writes the
+// same bits.  Two memory round trips, no counter, no barrier, nothing to reset (epochs only move forward), and the
+// result does not depend on arrival order.
+// Each XCD has its own L2, so data that crosses workgroups goes through device-scope stores and loads (written through
+// to / read from the memory side).  A device-wide fence would also order them, but it writes back and invalidates the
+// whole L2 under the other workgroups' streaming loads.
+// Call from the first 32 threads of the workgroup (one wave), total = the row's partial sum over this split.
+__device__ __forceinline__ void split_k_finish(uint64_t* __restrict__ tagged, unsigned epoch, int gstrip, int splits, int split, int lane, float total, float* __restrict__ y, int row,
+	int N, const float* __restrict__ residual) {
+	uint64_t* mine = tagged + static_cast<int64_t>(gstrip) * splits * STRIP_ROWS + lane;
+	__hip_atomic_store(&mine[split * STRIP_ROWS], (static_cast<uint64_t>(epoch) << 32) | __float_as_uint(total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+	wait_stores_acknowledged();
+	bool all  = true;
+	float sum = 0.0f;
+	for (int sp0 = 0; sp0 < splits; sp0 += 8) { // every share requested before the first is waited for
+		uint64_t v[8];
+#pragma unroll
+		for (int u = 0; u < 8; ++u) {
+			v[u] = (sp0 + u < splits) ? __hip_atomic_load(&mine[(sp0 + u) * STRIP_ROWS], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+		}
+#pragma unroll
+		for (int u = 0; u < 8; ++u) {
+			if (sp0 + u < splits) {
+				all = all && static_cast<unsigned>(v[u] >> 32) == epoch;
+				sum += __uint_as_float(static_cast<uint32_t>(v[u]));
+			}
+		}
+	}
+	if (all && row < N) {
+		y[row] = residual ? sum + residual[row] : sum;
+	}
+}
+
+// Scratch of the K-split path (tagged partial sums) and of the fused FFN launch (the gate and up
 // projections' outputs and one "published" word per producer strip): one allocation per device, made on first use and
 // kept for the life of the process.  Calls that overlap on one GPU (different streams) and both use it race on it.
 constexpr int GEMV_MAX_SPLIT_UNITS	= 8192; // strips * splits when splits > 1
 constexpr int GEMV_MAX_SPLIT_STRIPS = 512;
 constexpr int FFN_MAX_HIDDEN		= 65536; // rows of the gate / up projections in a fused FFN launch
 struct gemv_scratch {
-	float* partials	   = nullptr;
-	unsigned* counters = nullptr;
+	uint64_t* tagged   = nullptr; // [GEMV_MAX_SPLIT_UNITS][32] {epoch, partial sum}
 	float* gate_up	   = nullptr; // [2][FFN_MAX_HIDDEN]: the gate and up outputs (kept for inspection only)
 	uint32_t* act_q	   = nullptr; // [FFN_MAX_HIDDEN / 32][8]: the quantized activation of the down projection, 8 dwords per block
 	float* act_d	   = nullptr; // [FFN_MAX_HIDDEN / 32]: its scales (the fp16-rounded value, widened)
