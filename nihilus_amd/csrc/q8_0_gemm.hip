@@ -362,8 +362,13 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 	const uint8_t* a = static_cast<const uint8_t*>(Aq);
 	const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
 	if (tiled) {
-		if (M <= GEMM_SKINNY_MAX_M) {
-			return launch_gemm_skinny(W, Aq, C, sums, M, N, K, s); // few rows: weights are read once, the kernel is HBM-bound
+		// Few rows: the weights are read once and the kernel is HBM-bound.  Somewhat more rows than that, but so few
+		// 128-row x 32-row tiles that the tile kernel would leave most SIMDs with one wave or none (measured: it needs
+		// more than one workgroup per CU to pay): the same streaming kernel over groups of 64 rows, K split over the
+		// waves of a workgroup, the weights coming from cache after the first group.
+		const int64_t tile_workgroups = ((N + 127) / 128) * ((M + 31) / 32);
+		if (M <= GEMM_SKINNY_MAX_M || tile_workgroups <= 256) {
+			return launch_gemm_skinny(W, Aq, C, sums, M, N, K, s);
 		}
 		return launch_gemm_tiled(w, a, C, sums, m, n, k, s);
 	} else {

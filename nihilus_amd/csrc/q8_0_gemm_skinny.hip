@@ -40,6 +40,8 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 	const int splits = 1 << split_shift;
 	const int strip	 = static_cast<int>(blockIdx.x >> split_shift);
 	const int split	 = static_cast<int>(blockIdx.x) & (splits - 1);
+	const int mg	 = static_cast<int>(blockIdx.y); // group of MS activation strips (more than 32 * MS rows: the weights are read once per group, from cache after the first)
+	const int unit	 = mg * static_cast<int>(gridDim.x >> split_shift) + strip; // index of this (row group, weight strip) in the split scratch
 	const int slot	 = split * SK_WAVES + wave;
 	const int g0	 = slot * groups_per_slot + min(slot, groups_rem);
 	const int g1	 = g0 + groups_per_slot + (slot < groups_rem ? 1 : 0);
@@ -69,7 +71,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 				wd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
 #pragma unroll
 				for (int i = 0; i < MS; ++i) {
-					const uint8_t* am = A + macro_offset(i, gc + t, groups);
+					const uint8_t* am = A + macro_offset(mg * MS + i, gc + t, groups);
 #pragma unroll
 					for (int j = 0; j < GROUP_BLOCKS; ++j) {
 						aq[t][i][j] = *reinterpret_cast<const v4i*>(am + j * TILE_BYTES + 16 * lane);
@@ -96,7 +98,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 							const int n = strip * STRIP_ROWS + r;
 #pragma unroll
 							for (int e = 0; e < 16; ++e) {
-								const int m = i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+								const int m = (mg * MS + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 								if (m < M && n < N) {
 									sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + ((gc + t) * GROUP_BLOCKS + j)] = s[e];
 								}
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 			for (int i = 0; i < MS; ++i) {
 #pragma unroll
 				for (int e = 0; e < 16; ++e) {
-					const int m = i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+					const int m = (mg * MS + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 					if (m < M) {
 						C[static_cast<int64_t>(m) * N + n] = acc[i][e];
 					}
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 	}
 
 	// ---- K split over several workgroups: partial tiles through device-scope atomics, last arriver adds in split order ----
-	float* mine = partials + (static_cast<int64_t>(strip) * splits + split) * (MS * 16 * 64);
+	float* mine = partials + (static_cast<int64_t>(unit) * splits + split) * (MS * 16 * 64);
 	if (wave == 0) {
 #pragma unroll
 		for (int i = 0; i < MS; ++i) {
@@ -174,10 +176,10 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 	wait_stores_acknowledged();
 	__syncthreads();
 	if (tid == 0) {
-		const unsigned prev = __hip_atomic_fetch_add(&counters[strip], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		const unsigned prev = __hip_atomic_fetch_add(&counters[unit], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		const int last		= (prev == static_cast<unsigned>(splits - 1));
 		if (last) {
-			__hip_atomic_store(&counters[strip], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			__hip_atomic_store(&counters[unit], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		}
 		last_flag = last;
 	}
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 		for (int i = 0; i < MS; ++i) {
 			sum[i] = sk_v16f{ 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
 		}
-		const float* base = partials + static_cast<int64_t>(strip) * splits * (MS * 16 * 64) + lane;
+		const float* base = partials + static_cast<int64_t>(unit) * splits * (MS * 16 * 64) + lane;
 #pragma unroll
 		for (int i = 0; i < MS; ++i) {
 			for (int sp0 = 0; sp0 < splits; sp0 += 2) {
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 			}
 #pragma unroll
 			for (int e = 0; e < 16; ++e) {
-				const int m = i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+				const int m = (mg * MS + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 				if (m < M) {
 					C[static_cast<int64_t>(m) * N + n] = sum[i][e];
 				}
@@ -263,11 +265,13 @@ static hipError_t get_skinny_scratch(skinny_scratch* out) {
 }
 
 template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int groups, hipStream_t s) {
-	const int strips = (n + STRIP_ROWS - 1) / STRIP_ROWS;
-	int splits		 = 1;
+	const int strips   = (n + STRIP_ROWS - 1) / STRIP_ROWS;
+	const int m_groups = ((m + STRIP_ROWS - 1) / STRIP_ROWS + MS - 1) / MS;
+	const int units	   = strips * m_groups;
+	int splits		   = 1;
 	// The hand-off between workgroups costs a few microseconds, so K is split over workgroups only when a wave would
 	// otherwise walk more than four groups one after the other (few rows, long K: the down projections).
-	while (groups > 4 * SK_WAVES * splits && strips * splits * 2 <= SK_MAX_SPLIT_UNITS && strips <= SK_MAX_SPLIT_STRIPS) {
+	while (groups > 4 * SK_WAVES * splits && units * splits * 2 <= SK_MAX_SPLIT_UNITS && units <= SK_MAX_SPLIT_STRIPS) {
 		splits *= 2;
 	}
 	skinny_scratch sc;
@@ -282,7 +286,7 @@ template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8
 		++shift;
 	}
 	const int slots = splits * SK_WAVES, per_slot = groups / slots, rem = groups % slots;
-	const dim3 grid(static_cast<unsigned>(strips * splits)), block(SK_WAVES * 64);
+	const dim3 grid(static_cast<unsigned>(strips * splits), static_cast<unsigned>(m_groups)), block(SK_WAVES * 64);
 	if (sums) {
 		gemm_skinny_kernel<MS, true><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
 		return hipGetLastError();
@@ -294,7 +298,10 @@ hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* 
 	const uint8_t* w = static_cast<const uint8_t*>(W);
 	const uint8_t* a = static_cast<const uint8_t*>(Aq);
 	const int groups = static_cast<int>(K / GROUP_K);
-	if (M <= 32) {
+	// Two activation strips per workgroup halve the weight traffic per row, but only pay once the grid fills the chip
+	// without them: 64 rows against 128 weight strips are better off as 256 workgroups of one strip each.
+	const int64_t strips = (N + STRIP_ROWS - 1) / STRIP_ROWS, m_strips = (M + STRIP_ROWS - 1) / STRIP_ROWS;
+	if (m_strips <= 1 || strips * ((m_strips + 1) / 2) < 256) {
 		return launch_skinny_t<1>(w, a, C, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
 	}
 	return launch_skinny_t<2>(w, a, C, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
