@@ -16,8 +16,6 @@
 namespace nh {
 
 constexpr int SK_WAVES = 8;
-constexpr int SK_TILES = 1; // 128-quant groups per chunk: loads of one chunk are all in flight together; one keeps the
-                            // register count low enough for two workgroups per CU, so one computes while the other waits on loads
 
 typedef _Float16 sk_v4h __attribute__((ext_vector_type(4)));
 typedef float sk_v16f __attribute__((ext_vector_type(16)));
@@ -28,8 +26,8 @@ __device__ __forceinline__ v2u scale_slot(v2u four, int t) {
 	return v2u{ (t & 1) ? (dword >> 16) : (dword & 0xFFFFu), 0u };
 }
 
-template<int MS, bool DUMP>
-__global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums,
+template<int MS, bool DUMP, bool DB>
+__global__ __launch_bounds__(SK_WAVES * 64, (MS == 1 && !DB) ? 4 : 2) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums,
 	float* __restrict__ partials, unsigned* __restrict__ counters, int M, int N, int groups, int split_shift, int groups_per_slot, int groups_rem) {
 	__shared__ float red[SK_WAVES / 2][MS][16][64];
 	__shared__ int last_flag;
@@ -55,65 +53,89 @@ __global__ __launch_bounds__(SK_WAVES * 64, MS == 1 ? 2 : 1) void gemm_skinny_ke
 	}
 
 	const uint8_t* w_strip = W + macro_offset(strip, 0, groups);
-	for (int gc = g0; gc < g1; gc += SK_TILES) {
-		const int cnt = min(SK_TILES, g1 - gc);
-		// ---- every byte of the chunk in flight: weight tiles (HBM, non-temporal) and activation tiles (L2) ----
-		v4i wq[SK_TILES][GROUP_BLOCKS], aq[SK_TILES][MS][GROUP_BLOCKS];
-		v2u wd[SK_TILES], ad[SK_TILES][MS];
+	// One 128-quant group at a time per wave.  DB (a grid too small for two workgroups per CU): the next group's loads are
+	// issued before the current one is computed (two register sets).  That loop is written so that the number of loads in flight at every wait is a compile-time fact
+	// (loads complete in issue order, and a wait names how many later ones may stay outstanding): the steady-state body
+	// always issues a full set, the ragged end is peeled.
+	struct group_regs {
+		v4i wq[GROUP_BLOCKS], aq[MS][GROUP_BLOCKS];
+		v2u wd, ad[MS];
+	};
+	auto issue = [&](int g, group_regs& b) {
+		const uint8_t* macro = w_strip + static_cast<int64_t>(g) * MACRO_BYTES;
 #pragma unroll
-		for (int t = 0; t < SK_TILES; ++t) {
-			if (t < cnt) {
-				const uint8_t* macro = w_strip + static_cast<int64_t>(gc + t) * MACRO_BYTES;
+		for (int j = 0; j < GROUP_BLOCKS; ++j) {
+			b.wq[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+		}
+		b.wd = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
 #pragma unroll
-				for (int j = 0; j < GROUP_BLOCKS; ++j) {
-					wq[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
-				}
-				wd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+		for (int i = 0; i < MS; ++i) {
+			const uint8_t* am = A + macro_offset(mg * MS + i, g, groups);
 #pragma unroll
-				for (int i = 0; i < MS; ++i) {
-					const uint8_t* am = A + macro_offset(mg * MS + i, gc + t, groups);
+			for (int j = 0; j < GROUP_BLOCKS; ++j) {
+				b.aq[i][j] = *reinterpret_cast<const v4i*>(am + j * TILE_BYTES + 16 * lane);
+			}
+			b.ad[i] = *reinterpret_cast<const v2u*>(am + MACRO_D_OFFSET + 8 * r);
+		}
+	};
+	auto compute = [&](int g, const group_regs& b) {
+		// lanes 32..63 feed the k = 4..7 slots of the scale MFMA: zero
+		const v2u wdz = half ? v2u{ 0u, 0u } : b.wd;
 #pragma unroll
-					for (int j = 0; j < GROUP_BLOCKS; ++j) {
-						aq[t][i][j] = *reinterpret_cast<const v4i*>(am + j * TILE_BYTES + 16 * lane);
+		for (int j = 0; j < GROUP_BLOCKS; ++j) {
+			const v2u ws = scale_slot(wdz, j);
+#pragma unroll
+			for (int i = 0; i < MS; ++i) {
+				const sk_v16f zf = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+				const v16i zi	 = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+				const v16i s	 = __builtin_amdgcn_mfma_i32_32x32x32_i8(b.aq[i][j], b.wq[j], zi, 0, 0, 0);
+				if constexpr (DUMP) {
+					const int n = strip * STRIP_ROWS + r;
+#pragma unroll
+					for (int e = 0; e < 16; ++e) {
+						const int m = (mg * MS + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+						if (m < M && n < N) {
+							sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + (g * GROUP_BLOCKS + j)] = s[e];
+						}
 					}
-					ad[t][i] = *reinterpret_cast<const v2u*>(am + MACRO_D_OFFSET + 8 * r);
+				} else {
+					const v2u as	= scale_slot(half ? v2u{ 0u, 0u } : b.ad[i], j);
+					const sk_v16f p = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(sk_v4h, as), __builtin_bit_cast(sk_v4h, ws), zf, 0, 0, 0);
+#pragma unroll
+					for (int e = 0; e < 16; ++e) {
+						acc[i][e] = fmaf(static_cast<float>(s[e]), p[e], acc[i][e]);
+					}
 				}
 			}
 		}
-		// ---- MFMA per block, fold per block ----
-#pragma unroll
-		for (int t = 0; t < SK_TILES; ++t) {
-			if (t < cnt) {
-				// lanes 32..63 feed the k = 4..7 slots of the scale MFMA: zero
-				const v2u wdz = half ? v2u{ 0u, 0u } : wd[t];
-#pragma unroll
-				for (int j = 0; j < GROUP_BLOCKS; ++j) {
-					const v2u ws = scale_slot(wdz, j);
-#pragma unroll
-					for (int i = 0; i < MS; ++i) {
-						const sk_v16f zf = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-						const v16i zi	 = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-						const v16i s	 = __builtin_amdgcn_mfma_i32_32x32x32_i8(aq[t][i][j], wq[t][j], zi, 0, 0, 0);
-						if constexpr (DUMP) {
-							const int n = strip * STRIP_ROWS + r;
-#pragma unroll
-							for (int e = 0; e < 16; ++e) {
-								const int m = (mg * MS + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-								if (m < M && n < N) {
-									sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + ((gc + t) * GROUP_BLOCKS + j)] = s[e];
-								}
-							}
-						} else {
-							const v2u as	= scale_slot(half ? v2u{ 0u, 0u } : ad[t][i], j);
-							const sk_v16f p = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(sk_v4h, as), __builtin_bit_cast(sk_v4h, ws), zf, 0, 0, 0);
-#pragma unroll
-							for (int e = 0; e < 16; ++e) {
-								acc[i][e] = fmaf(static_cast<float>(s[e]), p[e], acc[i][e]);
-							}
-						}
-					}
-				}
-			}
+	};
+	if constexpr (!DB) {
+		// a grid of two or more workgroups per CU: one register set, the other workgroup computes while this one waits
+		for (int g = g0; g < g1; ++g) {
+			group_regs b;
+			issue(g, b);
+			__builtin_amdgcn_sched_barrier(0); // every load of the group before the first MFMA (left alone, the compiler interleaves them: measured slower)
+			compute(g, b);
+		}
+	} else if (g0 < g1) {
+		group_regs b0, b1;
+		issue(g0, b0);
+		int g = g0;
+		for (; g + 2 < g1; g += 2) { // at the top: b0 in flight
+			issue(g + 1, b1);
+			__builtin_amdgcn_sched_barrier(0);
+			compute(g, b0);
+			issue(g + 2, b0);
+			__builtin_amdgcn_sched_barrier(0);
+			compute(g + 1, b1);
+		}
+		if (g + 1 < g1) { // two groups left
+			issue(g + 1, b1);
+			__builtin_amdgcn_sched_barrier(0);
+			compute(g, b0);
+			compute(g + 1, b1);
+		} else { // one
+			compute(g, b0);
 		}
 	}
 	if constexpr (DUMP) {
@@ -288,10 +310,13 @@ template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8
 	const int slots = splits * SK_WAVES, per_slot = groups / slots, rem = groups % slots;
 	const dim3 grid(static_cast<unsigned>(strips * splits), static_cast<unsigned>(m_groups)), block(SK_WAVES * 64);
 	if (sums) {
-		gemm_skinny_kernel<MS, true><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+		gemm_skinny_kernel<MS, true, false><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+	if (static_cast<int64_t>(grid.x) * grid.y <= 256) { // at most one workgroup per CU: hide the load latency inside the wave
+		return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, true>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+	}
+	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, false>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
 }
 
 hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s) {
