@@ -61,7 +61,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
     ap.add_argument("--calibration-copies", type=int, default=0, help="run this many plain 64 MiB device copies first (a known-size kernel to scale hardware byte counters by)")
-    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover"], default="ffn_decode",
+    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover", "llama70b"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
     ap.add_argument("--ffn-mode", choices=["batch", "fused"], default="batch",
@@ -330,6 +330,48 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                 "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate", "data": "synthetic",
                 "config": {"workload": "nh_q8_0_mul_mat, fp32 activations [M x 4096] x Q8_0 W [4096x4096] and [14336x4096], activation quantize included, weights cache-resident "
                            "(17.8 / 62.4 MB against a 256 MB last-level cache): the GEMV -> GEMM crossover, not an HBM figure"}, "rows": rows}
+
+    if kind == "llama70b":
+        # BASELINE config 5: the LLaMA-3-70B projections at batched-decode sizes; weight sets are rotated so that
+        # each launch streams its matrix from HBM (the figure is weight bytes / time, the quantize launch included)
+        k70 = {"q_o": (8192, 8192), "k_v": (1024, 8192), "gate_up": (28672, 8192), "down": (8192, 28672), "lm_head": (128256, 8192)}
+        rows = []
+        for name, (n, k) in k70.items():
+            wbytes = n * (k // 32) * 34
+            copies = max(1, min(16, int(1.2e9 // wbytes)))
+            ws = []
+            for c_i in range(copies):
+                b = q8_0.fill_weight_blocks(11 + c_i, n, k)
+                ws.append(q8_0.tile(b, n, k))
+                del b
+            for m in (1, 4, 16, 64):
+                xm = q8_0.fill_activations(m, m * k).reshape(m, k)
+                ws_bytes = max(256, lib.nh_q8_0_mul_mat_workspace_bytes(m, k))
+                wsp = torch.empty(ws_bytes, dtype=torch.uint8, device=xm.device)
+                c = torch.empty((m, n), dtype=torch.float32, device=xm.device)
+                it = [0]
+
+                def fn():
+                    w = ws[it[0] % copies]
+                    it[0] += 1
+                    _lib.check("nh_q8_0_mul_mat", lib.nh_q8_0_mul_mat(w.data_ptr(), xm.data_ptr(), c.data_ptr(), m, n, k, wsp.data_ptr(), ws_bytes, stream))
+
+                for _ in range(warmup):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    fn()
+                torch.cuda.synchronize()
+                sec = (time.perf_counter() - t0) / steps
+                rows.append({"projection": name, "M": m, "N": n, "K": k, "us": round(sec * 1e6, 2), "weight_GBs": round(wbytes / sec / 1e9, 1),
+                             "pct_hbm": round(100 * wbytes / sec / 1e9 / HBM_PEAK_GBS, 1), "TOPs": round(2.0 * m * n * k / sec / 1e12, 2)})
+            del ws
+            torch.cuda.empty_cache()
+        return {"metric": "Q8_0 mul_mat weight-streaming GB/s at LLaMA-3-70B projection shapes, batched decode", "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+                "higher_is_better": True, "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate", "data": "synthetic",
+                "config": {"workload": "nh_q8_0_mul_mat, fp32 activations [M x K] x Q8_0 W at the 70B shapes, M in {1, 4, 16, 64}, activation quantize included, "
+                           "weight sets rotated over > 1 GB (lm_head: one 1.1 GB matrix)"}, "rows": rows}
 
     if kind == "get_rows":
         n_rows = 128256  # LLaMA-3 vocabulary; token_embd.weight [4096 x 128256] Q8_0 = 558 MB, rows picked at random
