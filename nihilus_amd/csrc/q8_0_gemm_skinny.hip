@@ -16,7 +16,6 @@
 namespace nh {
 
 constexpr int SK_WAVES = 8;
-
 typedef _Float16 sk_v4h __attribute__((ext_vector_type(4)));
 typedef float sk_v16f __attribute__((ext_vector_type(16)));
 
@@ -26,8 +25,8 @@ __device__ __forceinline__ v2u scale_slot(v2u four, int t) {
 	return v2u{ (t & 1) ? (dword >> 16) : (dword & 0xFFFFu), 0u };
 }
 
-template<int MS, bool DUMP, bool DB>
-__global__ __launch_bounds__(SK_WAVES * 64, (MS == 1 && !DB) ? 4 : 2) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums,
+template<int MS, bool DUMP, int GC>
+__global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums,
 	float* __restrict__ partials, unsigned* __restrict__ counters, int M, int N, int groups, int split_shift, int groups_per_slot, int groups_rem) {
 	__shared__ float red[SK_WAVES / 2][MS][16][64];
 	__shared__ int last_flag;
@@ -53,34 +52,46 @@ __global__ __launch_bounds__(SK_WAVES * 64, (MS == 1 && !DB) ? 4 : 2) void gemm_
 	}
 
 	const uint8_t* w_strip = W + macro_offset(strip, 0, groups);
-	// One 128-quant group at a time per wave.  DB (a grid too small for two workgroups per CU): the next group's loads are
-	// issued before the current one is computed (two register sets).  That loop is written so that the number of loads in flight at every wait is a compile-time fact
-	// (loads complete in issue order, and a wait names how many later ones may stay outstanding): the steady-state body
-	// always issues a full set, the ragged end is peeled.
-	struct group_regs {
-		v4i wq[GROUP_BLOCKS], aq[MS][GROUP_BLOCKS];
-		v2u wd, ad[MS];
+	struct w_regs {
+		v4i q[GROUP_BLOCKS];
+		v2u d;
 	};
-	auto issue = [&](int g, group_regs& b) {
+	struct a_regs {
+		v4i q[MS][GROUP_BLOCKS];
+		v2u d[MS];
+	};
+	auto issue_w = [&](int g, w_regs& b) {
 		const uint8_t* macro = w_strip + static_cast<int64_t>(g) * MACRO_BYTES;
 #pragma unroll
 		for (int j = 0; j < GROUP_BLOCKS; ++j) {
-			b.wq[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+			b.q[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
 		}
-		b.wd = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+		b.d = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+	};
+	// Activation rows beyond M are zero padding in the tiled operand.  Their lanes all read the strip's last row instead of
+	// their own (zeros as well, since a strip with any padding ends in it): one cache line per load instead of one per four
+	// lanes, so a batch of 4 rows costs a fraction of the cache traffic of a full strip, with no extra registers or branches.
+	int a_q_off[MS], a_d_off[MS];
+#pragma unroll
+	for (int i = 0; i < MS; ++i) {
+		const bool real = (mg * MS + i) * STRIP_ROWS + r < M;
+		a_q_off[i]		= real ? 16 * lane : 16 * (STRIP_ROWS - 1);
+		a_d_off[i]		= real ? 8 * r : 8 * (STRIP_ROWS - 1);
+	}
+	auto issue_a = [&](int g, a_regs& b) {
 #pragma unroll
 		for (int i = 0; i < MS; ++i) {
 			const uint8_t* am = A + macro_offset(mg * MS + i, g, groups);
 #pragma unroll
 			for (int j = 0; j < GROUP_BLOCKS; ++j) {
-				b.aq[i][j] = *reinterpret_cast<const v4i*>(am + j * TILE_BYTES + 16 * lane);
+				b.q[i][j] = *reinterpret_cast<const v4i*>(am + j * TILE_BYTES + a_q_off[i]);
 			}
-			b.ad[i] = *reinterpret_cast<const v2u*>(am + MACRO_D_OFFSET + 8 * r);
+			b.d[i] = *reinterpret_cast<const v2u*>(am + MACRO_D_OFFSET + a_d_off[i]);
 		}
 	};
-	auto compute = [&](int g, const group_regs& b) {
+	auto compute = [&](int g, const w_regs& w, const a_regs& a) {
 		// lanes 32..63 feed the k = 4..7 slots of the scale MFMA: zero
-		const v2u wdz = half ? v2u{ 0u, 0u } : b.wd;
+		const v2u wdz = half ? v2u{ 0u, 0u } : w.d;
 #pragma unroll
 		for (int j = 0; j < GROUP_BLOCKS; ++j) {
 			const v2u ws = scale_slot(wdz, j);
@@ -88,7 +99,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, (MS == 1 && !DB) ? 4 : 2) void gemm_
 			for (int i = 0; i < MS; ++i) {
 				const sk_v16f zf = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
 				const v16i zi	 = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-				const v16i s	 = __builtin_amdgcn_mfma_i32_32x32x32_i8(b.aq[i][j], b.wq[j], zi, 0, 0, 0);
+				const v16i s	 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a.q[i][j], w.q[j], zi, 0, 0, 0);
 				if constexpr (DUMP) {
 					const int n = strip * STRIP_ROWS + r;
 #pragma unroll
@@ -99,7 +110,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, (MS == 1 && !DB) ? 4 : 2) void gemm_
 						}
 					}
 				} else {
-					const v2u as	= scale_slot(half ? v2u{ 0u, 0u } : b.ad[i], j);
+					const v2u as	= scale_slot(half ? v2u{ 0u, 0u } : a.d[i], j);
 					const sk_v16f p = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(sk_v4h, as), __builtin_bit_cast(sk_v4h, ws), zf, 0, 0, 0);
 #pragma unroll
 					for (int e = 0; e < 16; ++e) {
@@ -109,33 +120,26 @@ __global__ __launch_bounds__(SK_WAVES * 64, (MS == 1 && !DB) ? 4 : 2) void gemm_
 			}
 		}
 	};
-	if constexpr (!DB) {
-		// a grid of two or more workgroups per CU: one register set, the other workgroup computes while this one waits
-		for (int g = g0; g < g1; ++g) {
-			group_regs b;
-			issue(g, b);
-			__builtin_amdgcn_sched_barrier(0); // every load of the group before the first MFMA (left alone, the compiler interleaves them: measured slower)
-			compute(g, b);
+	// GC groups per step: all their loads are issued, then waited for together (loads complete in issue order, so a
+	// short-latency activation load queued behind a weight load returns no earlier than it: prefetching one kind deeper
+	// than the other buys nothing), then computed.  More groups per step = more bytes in flight per wave.
+	for (int g = g0; g < g1; g += GC) {
+		w_regs w[GC];
+		a_regs a[GC];
+#pragma unroll
+		for (int c = 0; c < GC; ++c) {
+			issue_w(min(g + c, g1 - 1), w[c]); // past the end: the last group again (a cache hit, never used) so that the waits stay countable
 		}
-	} else if (g0 < g1) {
-		group_regs b0, b1;
-		issue(g0, b0);
-		int g = g0;
-		for (; g + 2 < g1; g += 2) { // at the top: b0 in flight
-			issue(g + 1, b1);
-			__builtin_amdgcn_sched_barrier(0);
-			compute(g, b0);
-			issue(g + 2, b0);
-			__builtin_amdgcn_sched_barrier(0);
-			compute(g + 1, b1);
+#pragma unroll
+		for (int c = 0; c < GC; ++c) {
+			issue_a(min(g + c, g1 - 1), a[c]);
 		}
-		if (g + 1 < g1) { // two groups left
-			issue(g + 1, b1);
-			__builtin_amdgcn_sched_barrier(0);
-			compute(g, b0);
-			compute(g + 1, b1);
-		} else { // one
-			compute(g, b0);
+		__builtin_amdgcn_sched_barrier(0); // every load of the step before the first MFMA (left alone, the compiler interleaves them: measured slower)
+#pragma unroll
+		for (int c = 0; c < GC; ++c) {
+			if (c == 0 || g + c < g1) {
+				compute(g + c, w[c], a[c]);
+			}
 		}
 	}
 	if constexpr (DUMP) {
@@ -310,13 +314,10 @@ template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8
 	const int slots = splits * SK_WAVES, per_slot = groups / slots, rem = groups % slots;
 	const dim3 grid(static_cast<unsigned>(strips * splits), static_cast<unsigned>(m_groups)), block(SK_WAVES * 64);
 	if (sums) {
-		gemm_skinny_kernel<MS, true, false><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+		gemm_skinny_kernel<MS, true, 1><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
 		return hipGetLastError();
 	}
-	if (static_cast<int64_t>(grid.x) * grid.y <= 256) { // at most one workgroup per CU: hide the load latency inside the wave
-		return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, true>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
-	}
-	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, false>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, 2>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
 }
 
 hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s) {
