@@ -450,8 +450,8 @@ int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K) {
 	if (M < 0 || K < 0 || K % nh::GROUP_K != 0) {
 		return NH_ERR_SHAPE;
 	}
-	if (M <= 1) {
-		return 0; // one row: the quantize happens inside the mat-vec kernel, nothing is staged in memory
+	if (M <= nh::GEMV_ROWS_MAX) {
+		return 0; // a few rows: the quantize happens inside the mat-vec kernel, nothing is staged in memory
 	}
 	return (nh_q8_0_tiled_bytes(M, K) + 255) / 256 * 256;
 }
@@ -469,6 +469,12 @@ int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, in
 	}
 	if (M == 1) {
 		return nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream); // quantize fused into the mat-vec: the workspace stays unused
+	}
+	if (M <= nh::GEMV_ROWS_MAX && K > 0) { // a few rows: the same streaming kernel with M dot products per weight tile
+		NH_REQUIRE(W_tiled && y, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(W_tiled) && aligned16(y), NH_ERR_ALIGNMENT);
+		NH_TRY(require_device());
+		return from_hip(nh::launch_gemv_rows(W_tiled, x, y, M, N, K, as_stream(stream)));
 	}
 	NH_TRY(nh_q8_0_quantize_tiled(x, workspace, M, K, stream));
 	return nh_q8_0_gemm_tiled(W_tiled, workspace, y, M, N, K, stream);

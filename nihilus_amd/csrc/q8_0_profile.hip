@@ -171,6 +171,15 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 			i += g;
 			continue;
 		}
+		if (op.M <= nh::GEMV_ROWS_MAX) {
+			// two or three rows: still the mat-vec kernel (one dot product per row), quantize inside, no workspace
+			const int rc = nh_q8_0_mul_mat(op.W_tiled, op.x, op.y, op.M, op.N, op.K, nullptr, 0, stream);
+			if (rc != NH_OK) {
+				return rc;
+			}
+			++i;
+			continue;
+		}
 		const bool reuse = op.reuse_quantized_x && quantized_x == op.x && quantized_m == op.M && quantized_k == op.K;
 		if (!reuse) {
 			const int rc = nh_q8_0_quantize_tiled(op.x, workspace, op.M, op.K, stream);

@@ -61,6 +61,57 @@ def test_mul_mat_fused(q8, oracle):
         assert rel_l2(got, want) <= REL_L2_TOL
 
 
+@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (14336, 4096), (33, 128), (100, 1024), (8192, 28672), (1024, 8192), (40000, 8192), (64, 128 * 70)])
+def test_mul_mat_few_rows(q8, oracle, n, k):
+    # 2 or 3 activation rows: the streaming mat-vec with one dot product per row and weight tile, quantize inside the kernel
+    # (unsplit, K split over workgroups, chunked walk, ragged N); no workspace is needed there.  4 rows: the MFMA kernel.
+    w = oracle.fill_weights(n + k, n, k)
+    wt = q8.tile(to_dev(w), n, k)
+    for m in (2, 3, 4):
+        assert (q8._lib.lib().nh_q8_0_mul_mat_workspace_bytes(m, k) == 0) == (m <= 3)
+        x = oracle.fill_activations(m + n, m * k).reshape(m, k)
+        if m == 3:
+            x[1] = 0.0  # an all-zero row: d = 0, every quant 0
+            x[2, ::2] *= 1e-3
+        aq = oracle.quantize_rows(x)
+        want = oracle.gemm(w, aq, m, n, k, threads=8) if (k // 32) % 16 == 0 else oracle.gemm(w, aq, m, n, k)
+        got = to_host(q8.mul_mat(wt, to_dev(x), n, k))
+        assert got.shape == (m, n)
+        for i in range(m):
+            assert rel_l2(got[i], want[i]) <= REL_L2_TOL, (m, i)
+        # each row is the mat-vec of that row: same kernel family, same fixed order -> same bits when the K cut is the same
+        y0 = to_host(q8.gemv_f32(wt, to_dev(x[0]), n, k))
+        assert rel_l2(got[0], y0) < 2e-6
+
+
+def test_mul_mat_batch_mixed_rows(q8, oracle):
+    # one native call, five projections: two mat-vecs sharing x (one launch), a 3-row op with no workspace use, two 8-row ops sharing the quantized x
+    import torch
+
+    from nihilus_amd import _lib
+
+    k, shapes = 1024, [(1, 256), (1, 96), (3, 160), (8, 256), (8, 64)]
+    x1 = oracle.fill_activations(1, k).reshape(1, k)
+    x3 = oracle.fill_activations(3, 3 * k).reshape(3, k)
+    x8 = oracle.fill_activations(8, 8 * k).reshape(8, k)
+    xs = {1: x1, 3: x3, 8: x8}
+    xd = {m: to_dev(v) for m, v in xs.items()}
+    ops = (_lib.MulMatOp * len(shapes))()
+    keep, want = [], []
+    for i, (m, n) in enumerate(shapes):
+        w = oracle.fill_weights(40 + i, n, k)
+        wt = q8.tile(to_dev(w), n, k)
+        y = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        keep += [wt, y]
+        ops[i] = _lib.MulMatOp(wt.data_ptr(), xd[m].data_ptr(), y.data_ptr(), m, n, k, 1 if i in (1, 4) else 0, 0)
+        want.append(oracle.gemm(w, oracle.quantize_rows(xs[m]), m, n, k, threads=4))
+    need = q8._lib.lib().nh_q8_0_mul_mat_workspace_bytes(8, k)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    _lib.check("nh_q8_0_mul_mat_batch", q8._lib.lib().nh_q8_0_mul_mat_batch(ops, len(shapes), ws.data_ptr(), need, torch.cuda.current_stream().cuda_stream))
+    for i in range(len(shapes)):
+        assert rel_l2(to_host(keep[2 * i + 1]), want[i]) <= REL_L2_TOL, i
+
+
 def test_gemm_extreme_quants(q8, oracle):
     m, n, k = 32, 32, 128
     nb = k // 32
