@@ -169,27 +169,36 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const uint8_t* __res
 //     at <= 128 VGPRs, four workgroups per CU, four waves per SIMD.  (A two-result-set, software-pipelined variant
 //     at two waves per SIMD measured 8 % slower: with so few waves the SIMD falls back to the lone-wave issue rate
 //     whenever one of them waits.)
-template<int TM, bool DUMP>
-__global__ __launch_bounds__(256, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums, int M, int N,
+template<int TM, bool DUMP, int KS = 1>
+__global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums, int M, int N,
 	int groups) {
 	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
 	constexpr int STAGE_BYTES = DATA_BYTES + 16;
-	__shared__ __align__(16) uint8_t lds[2 * STAGE_BYTES];
+	// KS = 2: the workgroup holds two sets of four waves; set kr walks groups [kr * groups / 2, (kr + 1) * groups / 2) with its
+	// own activation stages, and the second set's results are added to the first's through LDS at the end (fixed order).  A
+	// grid too small to give every SIMD its four waves gets them this way without a second pass over memory.
+	__shared__ __align__(16) uint8_t lds_all[KS][2 * STAGE_BYTES];
+	__shared__ float red[KS > 1 ? (KS - 1) * 4 * TM * 16 * 64 : 1];
 	typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 	typedef float v16f __attribute__((ext_vector_type(16)));
 
 	const int tid	   = threadIdx.x;
 	const int lane	   = tid & 63;
-	const int wave	   = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wave	   = wave_all & 3; // which of the workgroup's four weight strips
+	const int kr	   = wave_all >> 2; // which K range
+	uint8_t* lds	   = lds_all[kr];
+	const int g_len	   = groups / KS; // the host launches KS > 1 only when it divides
+	const int g_base   = kr * g_len;
 	const int half	   = lane >> 5;
 	const int m_strips = (M + 31) / 32;
 	const int n_strips = (N + 31) / 32;
 	const int ms0	   = blockIdx.y * TM;
 	const int ns	   = blockIdx.x * 4 + wave;
-	if (tid < 8) {
-		*reinterpret_cast<uint32_t*>(lds + (tid >> 2) * STAGE_BYTES + DATA_BYTES + 4 * (tid & 3)) = 0u;
+	if ((tid & 255) < 8) {
+		*reinterpret_cast<uint32_t*>(lds + ((tid & 255) >> 2) * STAGE_BYTES + DATA_BYTES + 4 * (tid & 3)) = 0u;
 	}
-	const uint8_t* w_src = W + macro_offset(min(ns, n_strips - 1), 0, groups);
+	const uint8_t* w_src = W + macro_offset(min(ns, n_strips - 1), g_base, groups);
 	struct w_regs {
 		v4i q[GROUP_BLOCKS];
 		v2u d;
@@ -209,11 +218,11 @@ __global__ __launch_bounds__(256, 4) void gemm_tiled_kernel(const uint8_t* __res
 #pragma unroll
 	for (int j = 0; j < TM; ++j) {
 		const int u = TM * wave + j;
-		a_src[j]	= A + macro_offset(min(ms0 + u / 4, m_strips - 1), 0, groups) + (u % 4) * TILE_BYTES + 16 * lane;
+		a_src[j]	= A + macro_offset(min(ms0 + u / 4, m_strips - 1), g_base, groups) + (u % 4) * TILE_BYTES + 16 * lane;
 		a_dst[j]	= (u / 4) * MACRO_BYTES + (u % 4) * TILE_BYTES + 16 * lane;
 	}
 	const bool sc_copier   = wave < TM;
-	const uint8_t* sc_src = A + macro_offset(min(ms0 + min(wave, TM - 1), m_strips - 1), 0, groups) + MACRO_D_OFFSET + 4 * lane;
+	const uint8_t* sc_src = A + macro_offset(min(ms0 + min(wave, TM - 1), m_strips - 1), g_base, groups) + MACRO_D_OFFSET + 4 * lane;
 	const int sc_dst	   = min(wave, TM - 1) * MACRO_BYTES + MACRO_D_OFFSET + 4 * lane;
 	struct a_regs {
 		v4i q[TM];
@@ -252,7 +261,7 @@ __global__ __launch_bounds__(256, 4) void gemm_tiled_kernel(const uint8_t* __res
 	stash_a(0, pre);
 	__syncthreads();
 	auto trip = [&](int g, w_regs& cur, w_regs& nxt) {
-		const bool more = g + 1 < groups;
+		const bool more = g + 1 < g_len;
 		if (more) {
 			fetch_w(g + 1, nxt);
 			fetch_a(g + 1, pre);
@@ -279,7 +288,7 @@ __global__ __launch_bounds__(256, 4) void gemm_tiled_kernel(const uint8_t* __res
 					for (int e = 0; e < 16; ++e) {
 						const int m = (ms0 + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 						if (m < M && n < N) {
-							sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + g * GROUP_BLOCKS + t] = sv[e];
+							sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + (g_base + g) * GROUP_BLOCKS + t] = sv[e];
 						}
 					}
 				} else {
@@ -297,10 +306,38 @@ __global__ __launch_bounds__(256, 4) void gemm_tiled_kernel(const uint8_t* __res
 		}
 		__syncthreads();
 	};
-	for (int g = 0; g < groups; g += 2) {
+	for (int g = 0; g < g_len; g += 2) {
 		trip(g, wa, wb);
-		if (g + 1 < groups) {
+		if (g + 1 < g_len) {
 			trip(g + 1, wb, wa);
+		}
+	}
+	if constexpr (KS > 1 && !DUMP) {
+		// the second set parks its tiles, the first adds them
+		if (kr > 0) {
+			float* mine = red + ((kr - 1) * 4 + wave) * (TM * 16 * 64);
+#pragma unroll
+			for (int i = 0; i < TM; ++i) {
+#pragma unroll
+				for (int e = 0; e < 16; ++e) {
+					mine[(i * 16 + e) * 64 + lane] = acc[i][e];
+				}
+			}
+		}
+		__syncthreads();
+		if (kr > 0) {
+			return;
+		}
+#pragma unroll
+		for (int k = 1; k < KS; ++k) {
+			const float* theirs = red + ((k - 1) * 4 + wave) * (TM * 16 * 64);
+#pragma unroll
+			for (int i = 0; i < TM; ++i) {
+#pragma unroll
+				for (int e = 0; e < 16; ++e) {
+					acc[i][e] += theirs[(i * 16 + e) * 64 + lane];
+				}
+			}
 		}
 	}
 	if constexpr (!DUMP) {
@@ -325,6 +362,10 @@ template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const u
 	if (sums) {
 		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, sums, m, n, groups);
 		return hipGetLastError();
+	}
+	// a grid that leaves SIMDs short of their four waves: two K sets inside the workgroup (8 waves) make up for it
+	if (static_cast<int64_t>(grid.x) * grid.y * 8 <= 4096 && groups % 2 == 0 && groups >= 8) {
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2>, grid, dim3(512), 0, s, w, a, C, sums, m, n, groups);
 	}
 	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false>, grid, dim3(256), 0, s, w, a, C, sums, m, n, groups);
 }
