@@ -10,7 +10,7 @@ from helpers import REL_L2_TOL, random_blocks, rel_l2, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336), (1024, 4096), (96, 512), (33, 128), (1, 128), (31, 256), (257, 8192), (8192, 28672), (1024, 8192), (100, 40960)]
+SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336), (1024, 4096), (128256, 4096), (96, 512), (33, 128), (1, 128), (31, 256), (257, 8192), (8192, 28672), (1024, 8192), (100, 40960)]
 
 
 def _inputs(oracle, n, k, seed):
