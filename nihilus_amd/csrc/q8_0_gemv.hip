@@ -115,7 +115,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* 
 //     depend on arrival order;
 //   * up to three weight matrices that share K and the activation row (q/k/v, gate/up) run as one launch:
 //     a bigger launch amortises the ramp-up and the tail.
-template<int TILES, bool XF32, int DUMP, bool LOOP, bool NORM>
+//   * RS > 1: a strip is shared by RS workgroups that own 32 / RS of its rows each and all of K (see gemv_chunk_n): how a
+//     matrix with few rows reaches every CU without partial sums.
+template<int TILES, bool XF32, int DUMP, bool LOOP, bool NORM, int RS = 1>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, uint64_t* __restrict__ tagged,
 	unsigned epoch, int groups, int split_shift, int groups_per_slot, int groups_rem, const float* __restrict__ norm_w, float norm_eps) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K]; // each wave's activation quants, block jj at 32*jj
@@ -126,9 +128,10 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	const int tid	 = threadIdx.x;
 	const int lane	 = tid & 63;
 	const int wave	 = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform by construction: keep it (and all that follows from it) scalar
-	const int splits = 1 << split_shift; // a power of two: no integer division anywhere on the way to the first load
-	const int gstrip = static_cast<int>(blockIdx.x >> split_shift); // strip index over all segments
-	const int split	 = static_cast<int>(blockIdx.x) & (splits - 1);
+	const int splits  = RS > 1 ? 1 : 1 << split_shift; // a power of two: no integer division anywhere on the way to the first load
+	const int gstrip  = RS > 1 ? static_cast<int>(blockIdx.x / RS) : static_cast<int>(blockIdx.x >> split_shift); // strip index over all segments
+	const int split	  = RS > 1 ? 0 : static_cast<int>(blockIdx.x) & (splits - 1);
+	const int rowpart = RS > 1 ? static_cast<int>(blockIdx.x % RS) : 0; // which 32 / RS rows of the strip
 	const int sidx	 = (gstrip >= seg.strip_end[0]) + (gstrip >= seg.strip_end[1]);
 	const int strip	 = gstrip - (sidx == 0 ? 0 : seg.strip_end[sidx - 1]);
 	const int N		 = seg.rows[sidx];
@@ -147,11 +150,11 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	}
 	if constexpr (!LOOP) {
 		// the host picked splits so that g1 - g0 <= TILES: straight-line code, every load of the wave in flight at once
-		acc = gemv_chunk<TILES, XF32, DUMP, NORM>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm);
+		acc = gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm, rowpart);
 	} else {
 		// K too long for that within the host's scratch limits: walk the range in chunks of TILES groups
 		for (int gc = g0; gc < g1; gc += TILES) {
-			acc += gemv_chunk<TILES, XF32, DUMP, NORM>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm);
+			acc += gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm, rowpart);
 			__builtin_amdgcn_wave_barrier(); // the next chunk overwrites this wave's LDS slice
 		}
 	}
@@ -162,17 +165,23 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	// ---- one reduction per workgroup, fixed order ----
 	red[wave][lane] = acc;
 	__syncthreads();
-	float total = 0.0f;
-	if (tid < STRIP_ROWS) {
+	constexpr int PART_ROWS = STRIP_ROWS / RS; // rows this workgroup owns: 64 / PART_ROWS lanes of every wave hold a share of each
+	float total				= 0.0f;
+	if (tid < PART_ROWS) {
 #pragma unroll
 		for (int w = 0; w < GEMV_WAVES; ++w) {
-			total += red[w][tid] + red[w][32 + tid];
+			float part = 0.0f; // this wave's shares of the row, then the waves in order
+#pragma unroll
+			for (int c = 0; c < 64 / PART_ROWS; ++c) {
+				part += red[w][c * PART_ROWS + tid];
+			}
+			total += part;
 		}
 	}
-	const int row = strip * STRIP_ROWS + tid;
+	const int row = strip * STRIP_ROWS + rowpart * PART_ROWS + tid;
 	float* y	  = seg.y[sidx];
 	if (splits == 1) {
-		if (tid < STRIP_ROWS && row < N) {
+		if (tid < PART_ROWS && row < N) {
 			y[row] = total;
 		}
 		return;
@@ -225,31 +234,48 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	return hipSuccess;
 }
 
-template<int TILES, bool XF32, bool LOOP, bool NORM> static hipError_t launch_gemv_tiled_n(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
-	const dim3 grid(static_cast<unsigned>(p.strips * p.splits)), block(GEMV_WAVES * 64);
-	int shift = 0;
-	while ((1 << shift) < p.splits) {
-		++shift;
+template<int TILES, bool XF32, bool LOOP, bool NORM, int RS = 1> static hipError_t launch_gemv_tiled_n(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
+	const dim3 grid(static_cast<unsigned>(p.strips * p.splits * RS)), block(GEMV_WAVES * 64);
+	if constexpr (RS > 1) { // row split (unsplit K, production only): RS workgroups per strip, nothing handed over
+		const int per_slot = p.groups / GEMV_WAVES, rem = p.groups % GEMV_WAVES;
+		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM, RS>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, 0, per_slot, rem, norm_w, norm_eps);
+	} else {
+		int shift = 0;
+		while ((1 << shift) < p.splits) {
+			++shift;
+		}
+		const int slots = p.splits * GEMV_WAVES, per_slot = p.groups / slots, rem = p.groups % slots;
+		if (dump_mode == DUMP_SUMS) {
+			gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+			return hipGetLastError();
+		}
+		if (dump_mode == DUMP_X) {
+			gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+			return hipGetLastError();
+		}
+		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 	}
-	const int slots = p.splits * GEMV_WAVES, per_slot = p.groups / slots, rem = p.groups % slots;
-	if (dump_mode == DUMP_SUMS) {
-		gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
-		return hipGetLastError();
-	}
-	if (dump_mode == DUMP_X) {
-		gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
-		return hipGetLastError();
-	}
-	return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
 }
 
-template<int TILES, bool XF32, bool LOOP> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
+template<int TILES, bool XF32, bool LOOP, int RS = 1> static hipError_t launch_gemv_tiled_t(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
 	if constexpr (XF32) {
 		if (norm_w) {
-			return launch_gemv_tiled_n<TILES, XF32, LOOP, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
+			return launch_gemv_tiled_n<TILES, XF32, LOOP, true, RS>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 		}
 	}
-	return launch_gemv_tiled_n<TILES, XF32, LOOP, false>(p, seg, x, dump, dump_mode, sc, nullptr, 0.0f, s);
+	return launch_gemv_tiled_n<TILES, XF32, LOOP, false, RS>(p, seg, x, dump, dump_mode, sc, nullptr, 0.0f, s);
+}
+
+// unsplit, at most four groups per wave, production: RS row parts per strip
+template<int RS, bool XF32> static hipError_t launch_gemv_tiled_rs(int tiles, const gemv_plan& p, const gemv_segments& seg, const void* x, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
+	switch (tiles) {
+		case 1:
+			return launch_gemv_tiled_t<1, XF32, false, RS>(p, seg, x, nullptr, DUMP_NONE, sc, norm_w, norm_eps, s);
+		case 2:
+			return launch_gemv_tiled_t<2, XF32, false, RS>(p, seg, x, nullptr, DUMP_NONE, sc, norm_w, norm_eps, s);
+		default:
+			return launch_gemv_tiled_t<4, XF32, false, RS>(p, seg, x, nullptr, DUMP_NONE, sc, norm_w, norm_eps, s);
+	}
 }
 
 static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, void* dump, int dump_mode, hipStream_t s,
@@ -280,6 +306,18 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 		return x_is_f32 ? launch_gemv_tiled_t<4, true, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s) : launch_gemv_tiled_t<4, false, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 	}
 	const int tiles = p.tiles <= 1 ? 1 : (p.tiles <= 2 ? 2 : 4);
+	if (dump_mode == DUMP_NONE && p.splits == 1) {
+		// Fewer strips than CUs (the 4096-row projections have 128, k/v 32): cut every strip into row parts so that the
+		// launch reaches RS times as many CUs.  What a single CU takes in per microsecond is limited, so half a chip
+		// cannot stream at the full HBM rate however many loads it has in flight.
+		const int rs = p.strips * 2 <= 256 ? (p.strips * 4 <= 256 ? 4 : 2) : 1;
+		if (rs == 4) {
+			return x_is_f32 ? launch_gemv_tiled_rs<4, true>(tiles, p, seg, x, sc, norm_w, norm_eps, s) : launch_gemv_tiled_rs<4, false>(tiles, p, seg, x, sc, norm_w, norm_eps, s);
+		}
+		if (rs == 2) {
+			return x_is_f32 ? launch_gemv_tiled_rs<2, true>(tiles, p, seg, x, sc, norm_w, norm_eps, s) : launch_gemv_tiled_rs<2, false>(tiles, p, seg, x, sc, norm_w, norm_eps, s);
+		}
+	}
 	if (x_is_f32) {
 		switch (tiles) {
 			case 1:

@@ -68,13 +68,25 @@ __device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, co
 // the compiler can wait for the activation slice alone, with the weight loads still in flight, only where it can
 // count the weight loads.  With a run-time count it has to wait for everything, and the quantizer runs after the last
 // weight byte has landed instead of under the stream.
-template<int TILES, int XMODE, int DUMP, bool NORM, int CNT>
+//
+// RS > 1 ("row split"): the workgroup owns only 32 / RS rows of its strip (part `rowpart`), and RS workgroups share the
+// strip.  A 1 KiB tile is two 512-byte halves (k 0..15 / 16..31) of 32 rows x 16 bytes, so the rows of one part are a
+// run of 512 / RS bytes in each half: whole 128-byte lines for RS <= 4.  One 16-byte-per-lane load then covers RS
+// blocks instead of one (a group takes 4 / RS loads per lane) and the lane's block and half follow from its number.
+// A matrix with fewer strips than the chip has CUs spreads over RS times as many of them this way, with nothing to
+// hand over between workgroups.
+template<int TILES, int XMODE, int DUMP, bool NORM, int CNT, int RS = 1>
 __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int groups,
-	int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2, const unsigned* __restrict__ flags, unsigned epoch, gemv_norm* norm) {
+	int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2, const unsigned* __restrict__ flags, unsigned epoch, gemv_norm* norm, int rowpart = 0) {
 	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
-	const int r	   = lane & 31;
-	const int half = lane >> 5;
+	static_assert(RS == 1 || RS == 2 || RS == 4, "a strip splits into 1, 2 or 4 row parts");
+	static_assert(RS == 1 || DUMP == DUMP_NONE, "the inspection variants run on whole strips");
+	constexpr int PART_ROWS = STRIP_ROWS / RS; // rows this workgroup owns
+	constexpr int W_LOADS	= GROUP_BLOCKS / RS; // 16-byte loads per lane and group
+	const int r	   = RS == 1 ? (lane & 31) : rowpart * PART_ROWS + (lane & (PART_ROWS - 1)); // row within the strip
+	const int half = RS == 1 ? (lane >> 5) : ((lane / PART_ROWS) & 1); // which 16 quants of its block the lane holds
+	const int blk0 = RS == 1 ? 0 : (lane / PART_ROWS) >> 1; // block of the lane's first load within the group; load j: blk0 + j * RS
 
 	// ---- 1. activation slice loads, issued first ----
 	constexpr int XQ_LOADS = (TILES * 34 + 63) / 64; // raw dwords of blocks [4*gc, 4*(gc+cnt)): 34 dwords per group
@@ -111,17 +123,19 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	}
 
 	// ---- 2. every weight byte of the chunk, in flight at once ----
-	v4i q[TILES][GROUP_BLOCKS];
+	v4i q[TILES][W_LOADS];
 	v2u dd[TILES];
 	if constexpr (DUMP != DUMP_X) {
 		const uint8_t* macro0 = w_strip + static_cast<int64_t>(gc) * MACRO_BYTES;
+		// byte offset of the lane's 16 quants inside its first tile: RS == 1 is the tile as stored (16 * lane)
+		const int lane_off = RS == 1 ? 16 * lane : blk0 * TILE_BYTES + half * (TILE_BYTES / 2) + 16 * r;
 #pragma unroll
 		for (int t = 0; t < TILES; ++t) {
 			if (t < cnt) {
 				const uint8_t* macro = macro0 + t * MACRO_BYTES;
 #pragma unroll
-				for (int j = 0; j < GROUP_BLOCKS; ++j) {
-					q[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+				for (int j = 0; j < W_LOADS; ++j) {
+					q[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * (RS * TILE_BYTES) + lane_off));
 				}
 				dd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
 			}
@@ -247,20 +261,33 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 #pragma unroll
 	for (int t = 0; t < TILES; ++t) {
 		if (t < cnt) {
-			const float dw[GROUP_BLOCKS] = { half_bits_to_float(static_cast<uint16_t>(dd[t].x & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].x >> 16)),
-				half_bits_to_float(static_cast<uint16_t>(dd[t].y & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].y >> 16)) };
+			if constexpr (RS == 1) {
+				const float dw[GROUP_BLOCKS] = { half_bits_to_float(static_cast<uint16_t>(dd[t].x & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].x >> 16)),
+					half_bits_to_float(static_cast<uint16_t>(dd[t].y & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[t].y >> 16)) };
 #pragma unroll
-			for (int j = 0; j < GROUP_BLOCKS; ++j) {
-				const int jj = t * GROUP_BLOCKS + j;
-				const v4i xv = *reinterpret_cast<const v4i*>(xs_q + jj * QK + 16 * half);
-				const int s	 = dot16(q[t][j], xv);
-				if constexpr (DUMP == DUMP_SUMS) {
-					const int full = s + __shfl_xor(s, 32);
-					if (half == 0 && row < N) {
-						static_cast<int32_t*>(dump)[static_cast<int64_t>(row) * (groups * GROUP_BLOCKS) + (gc * GROUP_BLOCKS + jj)] = full;
+				for (int j = 0; j < GROUP_BLOCKS; ++j) {
+					const int jj = t * GROUP_BLOCKS + j;
+					const v4i xv = *reinterpret_cast<const v4i*>(xs_q + jj * QK + 16 * half);
+					const int s	 = dot16(q[t][j], xv);
+					if constexpr (DUMP == DUMP_SUMS) {
+						const int full = s + __shfl_xor(s, 32);
+						if (half == 0 && row < N) {
+							static_cast<int32_t*>(dump)[static_cast<int64_t>(row) * (groups * GROUP_BLOCKS) + (gc * GROUP_BLOCKS + jj)] = full;
+						}
+					} else {
+						acc = fmaf(static_cast<float>(s), dw[j] * xs_d[jj], acc);
 					}
-				} else {
-					acc = fmaf(static_cast<float>(s), dw[j] * xs_d[jj], acc);
+				}
+			} else {
+#pragma unroll
+				for (int j = 0; j < W_LOADS; ++j) {
+					const int b		  = blk0 + j * RS; // the lane's block within the group
+					const int jj	  = t * GROUP_BLOCKS + b;
+					const uint32_t dp = (b & 2) ? dd[t].y : dd[t].x;
+					const float dw	  = half_bits_to_float(static_cast<uint16_t>((b & 1) ? (dp >> 16) : (dp & 0xFFFFu)));
+					const v4i xv	  = *reinterpret_cast<const v4i*>(xs_q + jj * QK + 16 * half);
+					const int s		  = dot16(q[t][j], xv);
+					acc				  = fmaf(static_cast<float>(s), dw * xs_d[jj], acc);
 				}
 			}
 		}
@@ -273,14 +300,14 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	return acc;
 }
 
-template<int TILES, int XMODE, int DUMP, bool NORM = false>
+template<int TILES, int XMODE, int DUMP, bool NORM = false, int RS = 1>
 __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
 	int groups, int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2 = nullptr, const unsigned* __restrict__ flags = nullptr, unsigned epoch = 0,
-	gemv_norm* norm = nullptr) {
+	gemv_norm* norm = nullptr, int rowpart = 0) {
 #define NH_CHUNK_CASE(C)                                                                                                                                              \
 	case C:                                                                                                                                                           \
 		if constexpr (C <= TILES) {                                                                                                                                   \
-			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0)>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm); \
+			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0), RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm, rowpart); \
 		}                                                                                                                                                             \
 		break;
 	switch (cnt) { // wave-uniform
@@ -292,7 +319,7 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 			break;
 	}
 #undef NH_CHUNK_CASE
-	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm); // an idle wave (still takes part in barriers)
+	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0, RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm, rowpart); // an idle wave (still takes part in barriers)
 }
 
 // K split over several workgroups: each publishes the 32 partial sums of its share, tagged with the launch's epoch
