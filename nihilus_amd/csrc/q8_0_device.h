@@ -184,6 +184,22 @@ __device__ __host__ __forceinline__ int64_t macro_offset(int64_t strip, int64_t 
 
 enum kernel_kind : int { KIND_QUANTIZE = 0, KIND_GEMV = 1, KIND_GEMM = 2, KIND_GET_ROWS = 3, KIND_COUNT = 4 };
 
+// The K range (in 128-quant groups) of one wave when a strip's `groups` are cut over `1 << split_shift` workgroups of `waves`
+// waves each: the groups go to the workgroups as evenly as they can (the first groups % splits take one more), then each
+// workgroup's share to its waves the same way.  Workgroups of one launch must not differ by more than a group: the CUs
+// that host the heavier ones finish last, and the launch with them (handing the remainder to the first waves of the
+// first workgroups instead cost the LLaMA-3-8B down projection 4 % of its time).  With one workgroup this is the cut
+// the fixed-order RMS-norm sum is defined on.  All operands are wave-uniform.
+__device__ __forceinline__ void wave_k_range(int groups, int split_shift, int split, int waves, int wave, int& g0, int& g1) {
+	const int splits  = 1 << split_shift;
+	const int s_q	  = groups >> split_shift, s_r = groups & (splits - 1);
+	const int s_start = split * s_q + min(split, s_r);
+	const int s_cnt	  = s_q + (split < s_r ? 1 : 0);
+	const int w_q = s_cnt / waves, w_r = s_cnt % waves;
+	g0 = s_start + wave * w_q + min(wave, w_r);
+	g1 = g0 + w_q + (wave < w_r ? 1 : 0);
+}
+
 // When timing is on for `kind` and the event pool has room, hands out an event pair for the next launch.
 bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop);
 

@@ -43,7 +43,7 @@ struct ffn_args {
 	int groups_p, groups_c; // K / 128, n_ff / 128
 	int producers; // n_ff / 32
 	int p_per_slot, p_rem; // a producer strip's K range over the 8 waves of one matrix
-	int split_shift, c_per_slot, c_rem; // a consumer strip's K range over splits * 16 waves
+	int split_shift; // a consumer strip's K range goes over (1 << split_shift) workgroups of 16 waves
 };
 
 template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
@@ -122,9 +122,8 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 	const int splits = 1 << a.split_shift;
 	const int gstrip = c >> a.split_shift;
 	const int split	 = c & (splits - 1);
-	const int slot	 = split * GEMV_WAVES + wave;
-	const int g0	 = slot * a.c_per_slot + min(slot, a.c_rem);
-	const int g1	 = g0 + a.c_per_slot + (slot < a.c_rem ? 1 : 0);
+	int g0, g1;
+	wave_k_range(a.groups_c, a.split_shift, split, GEMV_WAVES, wave, g0, g1);
 
 	const uint8_t* w_strip = a.w_down + macro_offset(gstrip, 0, a.groups_c);
 	const int row_l		   = gstrip * STRIP_ROWS + (lane & 31);
@@ -226,10 +225,7 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	while ((1 << shift) < splits) {
 		++shift;
 	}
-	const int slots		= splits * GEMV_WAVES;
 	a.split_shift		= shift;
-	a.c_per_slot		= a.groups_c / slots;
-	a.c_rem				= a.groups_c % slots;
 	const int tiles_p	= (a.groups_p + GEMV_WAVES / 2 - 1) / (GEMV_WAVES / 2);
 	const int tiles_c	= tiles_for(splits);
 	const int tiles		= tiles_p > tiles_c ? tiles_p : tiles_c;

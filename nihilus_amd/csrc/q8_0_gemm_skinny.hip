@@ -27,7 +27,7 @@ __device__ __forceinline__ v2u scale_slot(v2u four, int t) {
 
 template<int MS, bool DUMP, int GC>
 __global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums,
-	float* __restrict__ partials, unsigned* __restrict__ counters, int M, int N, int groups, int split_shift, int groups_per_slot, int groups_rem) {
+	float* __restrict__ partials, unsigned* __restrict__ counters, int M, int N, int groups, int split_shift) {
 	__shared__ float red[SK_WAVES / 2][MS][16][64];
 	__shared__ int last_flag;
 
@@ -39,9 +39,8 @@ __global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kerne
 	const int split	 = static_cast<int>(blockIdx.x) & (splits - 1);
 	const int mg	 = static_cast<int>(blockIdx.y); // group of MS activation strips (more than 32 * MS rows: the weights are read once per group, from cache after the first)
 	const int unit	 = mg * static_cast<int>(gridDim.x >> split_shift) + strip; // index of this (row group, weight strip) in the split scratch
-	const int slot	 = split * SK_WAVES + wave;
-	const int g0	 = slot * groups_per_slot + min(slot, groups_rem);
-	const int g1	 = g0 + groups_per_slot + (slot < groups_rem ? 1 : 0);
+	int g0, g1; // this wave's share of the strip's K range
+	wave_k_range(groups, split_shift, split, SK_WAVES, wave, g0, g1);
 	const int r		 = lane & 31;
 	const int half	 = lane >> 5;
 
@@ -316,13 +315,12 @@ template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8
 	while ((1 << shift) < splits) {
 		++shift;
 	}
-	const int slots = splits * SK_WAVES, per_slot = groups / slots, rem = groups % slots;
 	const dim3 grid(static_cast<unsigned>(strips * splits), static_cast<unsigned>(m_groups)), block(SK_WAVES * 64);
 	if (sums) {
-		gemm_skinny_kernel<MS, true, 1><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+		gemm_skinny_kernel<MS, true, 1><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, 2>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift, per_slot, rem);
+	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, 2>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift);
 }
 
 hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s) {

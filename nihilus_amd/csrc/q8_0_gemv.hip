@@ -119,7 +119,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* 
 //     matrix with few rows reaches every CU without partial sums.
 template<int TILES, bool XF32, int DUMP, bool LOOP, bool NORM, int RS = 1>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, uint64_t* __restrict__ tagged,
-	unsigned epoch, int groups, int split_shift, int groups_per_slot, int groups_rem, const float* __restrict__ norm_w, float norm_eps) {
+	unsigned epoch, int groups, int split_shift, const float* __restrict__ norm_w, float norm_eps) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K]; // each wave's activation quants, block jj at 32*jj
 	__shared__ float norm_red[16];
 	__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1]; // each wave's slice of the norm weights
@@ -135,9 +135,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	const int sidx	 = (gstrip >= seg.strip_end[0]) + (gstrip >= seg.strip_end[1]);
 	const int strip	 = gstrip - (sidx == 0 ? 0 : seg.strip_end[sidx - 1]);
 	const int N		 = seg.rows[sidx];
-	const int slot	 = split * GEMV_WAVES + wave; // this wave's share of the strip's K range:
-	const int g0	 = slot * groups_per_slot + min(slot, groups_rem); // groups = slots * groups_per_slot + groups_rem,
-	const int g1	 = g0 + groups_per_slot + (slot < groups_rem ? 1 : 0); // the first groups_rem slots take one extra
+	int g0, g1; // this wave's share of the strip's K range
+	wave_k_range(groups, RS > 1 ? 0 : split_shift, split, GEMV_WAVES, wave, g0, g1);
 
 	const uint8_t* w_strip = DUMP == DUMP_X ? nullptr : seg.W[sidx] + macro_offset(strip, 0, groups);
 	const int row_l		   = strip * STRIP_ROWS + (lane & 31);
@@ -237,23 +236,21 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 template<int TILES, bool XF32, bool LOOP, bool NORM, int RS = 1> static hipError_t launch_gemv_tiled_n(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
 	const dim3 grid(static_cast<unsigned>(p.strips * p.splits * RS)), block(GEMV_WAVES * 64);
 	if constexpr (RS > 1) { // row split (unsplit K, production only): RS workgroups per strip, nothing handed over
-		const int per_slot = p.groups / GEMV_WAVES, rem = p.groups % GEMV_WAVES;
-		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM, RS>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, 0, per_slot, rem, norm_w, norm_eps);
+		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM, RS>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, 0, norm_w, norm_eps);
 	} else {
 		int shift = 0;
 		while ((1 << shift) < p.splits) {
 			++shift;
 		}
-		const int slots = p.splits * GEMV_WAVES, per_slot = p.groups / slots, rem = p.groups % slots;
 		if (dump_mode == DUMP_SUMS) {
-			gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+			gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps);
 			return hipGetLastError();
 		}
 		if (dump_mode == DUMP_X) {
-			gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+			gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps);
 			return hipGetLastError();
 		}
-		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, per_slot, rem, norm_w, norm_eps);
+		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps);
 	}
 }
 

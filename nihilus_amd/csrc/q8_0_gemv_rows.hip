@@ -113,7 +113,7 @@ __device__ __forceinline__ void gemv_rows_chunk(const uint8_t* __restrict__ w_st
 // in 64 registers = two workgroups per CU; three take 65 and run as one, which measured faster than spilling to stay at two).
 template<int TILES, int MR, bool LOOP>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_rows_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, uint64_t* __restrict__ tagged, unsigned epoch,
-	int N, int groups, int split_shift, int groups_per_slot, int groups_rem) {
+	int N, int groups, int split_shift) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][MR][TILES * GROUP_K]; // each wave's quantized slices, block jj of row m at 32*jj
 	__shared__ float xs_d[GEMV_WAVES][MR][TILES * GROUP_BLOCKS];
 	__shared__ float red[MR][GEMV_WAVES][64];
@@ -123,9 +123,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_rows_kernel(const uint8_
 	const int splits = 1 << split_shift;
 	const int strip	 = static_cast<int>(blockIdx.x >> split_shift);
 	const int split	 = static_cast<int>(blockIdx.x) & (splits - 1);
-	const int slot	 = split * GEMV_WAVES + wave; // this wave's share of the strip's K range:
-	const int g0	 = slot * groups_per_slot + min(slot, groups_rem); // groups = slots * groups_per_slot + groups_rem,
-	const int g1	 = g0 + groups_per_slot + (slot < groups_rem ? 1 : 0); // the first groups_rem slots take one extra
+	int g0, g1; // this wave's share of the strip's K range
+	wave_k_range(groups, split_shift, split, GEMV_WAVES, wave, g0, g1);
 	const int64_t K	 = static_cast<int64_t>(groups) * GROUP_K;
 
 	const uint8_t* w_strip = W + macro_offset(strip, 0, groups);
@@ -175,8 +174,7 @@ template<int TILES, int MR, bool LOOP> static hipError_t launch_rows_n(const gem
 	while ((1 << shift) < p.splits) {
 		++shift;
 	}
-	const int slots = p.splits * GEMV_WAVES, per_slot = p.groups / slots, rem = p.groups % slots;
-	return launch_kernel(KIND_GEMV, gemv_rows_kernel<TILES, MR, LOOP>, grid, block, 0, s, W, x, y, sc.tagged, sc.epoch, N, p.groups, shift, per_slot, rem);
+	return launch_kernel(KIND_GEMV, gemv_rows_kernel<TILES, MR, LOOP>, grid, block, 0, s, W, x, y, sc.tagged, sc.epoch, N, p.groups, shift);
 }
 
 template<int MR> static hipError_t launch_rows_m(const gemv_plan& p, const uint8_t* W, const float* x, float* y, int N, const gemv_scratch& sc, hipStream_t s) {
