@@ -164,7 +164,9 @@ __device__ __forceinline__ float4 norm_mul4(float4 x, float scale, float4 w) {
 // so waiting for any register load issued after this one is enough.  lds_dst must be wave-uniform.
 __device__ __forceinline__ void load_global_to_lds_b128(const void* src, void* lds_dst) {
 	const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)(static_cast<char*>(lds_dst))));
-	asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory", "m0");
+	// the LDS address travels in M0, which the compiler may hold a value in: saved and put back around the transfer
+	uint32_t saved_m0;
+	asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0" : "=&s"(saved_m0) : "v"(src), "s"(lds_addr) : "memory");
 }
 
 // Blocks the wave until every memory operation it has issued, stores included, has been acknowledged.  Placed

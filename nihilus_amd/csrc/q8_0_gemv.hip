@@ -52,7 +52,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* 
 	const uint8_t* w_row	= W + row_c * row_bytes;
 
 	float acc = 0.0f;
-#pragma unroll 2
 	for (int g = wave; g < groups; g += WAVES) {
 		v4i q[GROUP_BLOCKS];
 		float dw[GROUP_BLOCKS];
