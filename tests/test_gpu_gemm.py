@@ -13,7 +13,7 @@ def _inputs(oracle, m, n, k, seed):
     return w, x, oracle.quantize_rows(x)
 
 
-@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (128, 14336, 4096), (32, 128, 128), (1, 128, 128), (8, 96, 256), (33, 65, 384), (130, 257, 512), (64, 4096, 14336)])
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (512, 14336, 4096), (128, 14336, 4096), (32, 128, 128), (1, 128, 128), (8, 96, 256), (33, 65, 384), (130, 257, 512), (64, 4096, 14336)])
 def test_gemm_tiled_and_blocks(q8, oracle, m, n, k):
     w, x, aq = _inputs(oracle, m, n, k, seed=m + n + k)
     want = oracle.gemm(w, aq, m, n, k, threads=8) if (k // 32) % 16 == 0 else oracle.gemm(w, aq, m, n, k)
