@@ -174,11 +174,11 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	int groups) {
 	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
 	constexpr int STAGE_BYTES = DATA_BYTES + 16;
-	// KS = 2: the workgroup holds two sets of four waves; set kr walks groups [kr * groups / 2, (kr + 1) * groups / 2) with its
-	// own activation stages, and the second set's results are added to the first's through LDS at the end (fixed order).  A
+	// KS > 1: the workgroup holds KS sets of four waves; set kr walks groups [kr * groups / KS, (kr + 1) * groups / KS) with its
+	// own activation stages, and the sets' results are added to the first's through LDS at the end (set order, fixed).  A
 	// grid too small to give every SIMD its four waves gets them this way without a second pass over memory.
 	__shared__ __align__(16) uint8_t lds_all[KS][2 * STAGE_BYTES];
-	__shared__ float red[KS > 1 ? (KS - 1) * 4 * TM * 16 * 64 : 1];
+	__shared__ float red[KS > 1 ? 4 * TM * 16 * 64 : 1];
 	typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 	typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -313,31 +313,35 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		}
 	}
 	if constexpr (KS > 1 && !DUMP) {
-		// the second set parks its tiles, the first adds them
-		if (kr > 0) {
-			float* mine = red + ((kr - 1) * 4 + wave) * (TM * 16 * 64);
-#pragma unroll
-			for (int i = 0; i < TM; ++i) {
-#pragma unroll
-				for (int e = 0; e < 16; ++e) {
-					mine[(i * 16 + e) * 64 + lane] = acc[i][e];
-				}
-			}
-		}
-		__syncthreads();
-		if (kr > 0) {
-			return;
-		}
+		// sets 1 .. KS-1 park their tiles one after the other in the same LDS buffer, set 0 adds them (set order, fixed)
+		float* slot = red + wave * (TM * 16 * 64);
 #pragma unroll
 		for (int k = 1; k < KS; ++k) {
-			const float* theirs = red + ((k - 1) * 4 + wave) * (TM * 16 * 64);
+			if (kr == k) {
 #pragma unroll
-			for (int i = 0; i < TM; ++i) {
+				for (int i = 0; i < TM; ++i) {
 #pragma unroll
-				for (int e = 0; e < 16; ++e) {
-					acc[i][e] += theirs[(i * 16 + e) * 64 + lane];
+					for (int e = 0; e < 16; ++e) {
+						slot[(i * 16 + e) * 64 + lane] = acc[i][e];
+					}
 				}
 			}
+			__syncthreads();
+			if (kr == 0) {
+#pragma unroll
+				for (int i = 0; i < TM; ++i) {
+#pragma unroll
+					for (int e = 0; e < 16; ++e) {
+						acc[i][e] += slot[(i * 16 + e) * 64 + lane];
+					}
+				}
+			}
+			if (k + 1 < KS) {
+				__syncthreads();
+			}
+		}
+		if (kr > 0) {
+			return;
 		}
 	}
 	if constexpr (!DUMP) {
@@ -363,8 +367,15 @@ template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const u
 		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, sums, m, n, groups);
 		return hipGetLastError();
 	}
-	// a grid that leaves SIMDs short of their four waves: two K sets inside the workgroup (8 waves) make up for it
-	if (static_cast<int64_t>(grid.x) * grid.y * 8 <= 4096 && groups % 2 == 0 && groups >= 8) {
+	// a grid that leaves SIMDs short of their four waves: K sets inside the workgroup (8 or 16 waves) make up for it
+	int ks = 1;
+	while (ks < 4 && static_cast<int64_t>(grid.x) * grid.y * 4 * ks * 2 <= 4096 && groups % (ks * 2) == 0 && groups / (ks * 2) >= 4) {
+		ks *= 2;
+	}
+	if (ks == 4) {
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4>, grid, dim3(1024), 0, s, w, a, C, sums, m, n, groups);
+	}
+	if (ks == 2) {
 		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2>, grid, dim3(512), 0, s, w, a, C, sums, m, n, groups);
 	}
 	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false>, grid, dim3(256), 0, s, w, a, C, sums, m, n, groups);
@@ -374,8 +385,11 @@ template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const u
 // the grid must give every SIMD at least two waves: 64-row workgroup tiles (half the LDS and L2 traffic per MFMA) when
 // that still leaves >= 512 workgroups, 32-row tiles otherwise.
 static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int k, hipStream_t s) {
-	const int64_t ms = (m + 31) / 32, ns4 = ((n + 31) / 32 + 3) / 4;
-	if (((ms + 1) / 2) * ns4 >= 1024) {
+	const int64_t ms = (m + 31) / 32;
+	// Two activation strips per wave whenever there are two: every weight tile fetched is used twice, which halves what a CU
+	// has to take in per MFMA (that intake, not the MFMA rate, bounds the one-strip form); the K sets below give back the
+	// waves the halved grid loses.
+	if (ms >= 2) {
 		return launch_gemm_tiled_t<2>(w, a, C, sums, m, n, k, s);
 	}
 	return launch_gemm_tiled_t<1>(w, a, C, sums, m, n, k, s);
