@@ -18,13 +18,26 @@ namespace nh {
 // gate and up projections' outputs), so the fp32 activation never makes a round trip through memory.
 template<bool TILED, bool SILU_MUL>
 __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, const float* __restrict__ u, uint8_t* __restrict__ out, int64_t M, int64_t rows_out, int64_t K) {
-	const int64_t nb	= K / QK;
-	const int64_t t		= static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-	const int64_t blk	= t >> 3; // block index over rows_out * nb
-	const int j			= static_cast<int>(t & 7); // which float4 of the block
-	const bool in_range = blk < rows_out * nb; // whole 8-lane groups agree, so the shuffles below stay converged per group
-	const int64_t m		= in_range ? blk / nb : 0;
-	const int64_t b		= in_range ? blk - m * nb : 0;
+	const int64_t nb = K / QK;
+	const int64_t t	 = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+	const int j		 = static_cast<int>(t & 7); // which float4 of the block
+	// Eight lanes per block either way.  Tiled output: a wave takes one block column of eight consecutive rows, so that its
+	// stores fill two whole 128-byte lines of the tile (8 rows x 16 bytes per half) instead of sixteen 16-byte pieces of
+	// eight different tiles; rows_out is a multiple of 32 there.  Blocks output: a wave takes eight consecutive blocks of a row.
+	int64_t m, b;
+	bool in_range;
+	if constexpr (TILED) {
+		const int64_t unit = t >> 6; // (8-row group, block column)
+		in_range		   = unit < (rows_out / 8) * nb;
+		const int64_t rg   = in_range ? unit / nb : 0;
+		b				   = in_range ? unit - rg * nb : 0;
+		m				   = rg * 8 + ((t >> 3) & 7);
+	} else {
+		const int64_t blk = t >> 3; // block index over rows_out * nb
+		in_range		  = blk < rows_out * nb; // whole 8-lane groups agree, so the shuffles below stay converged per group
+		m				  = in_range ? blk / nb : 0;
+		b				  = in_range ? blk - m * nb : 0;
+	}
 
 	float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 	if (in_range && m < M) {
@@ -51,7 +64,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
 			*reinterpret_cast<uint16_t*>(macro + MACRO_D_OFFSET + 8 * r + 2 * tq) = dh;
 		}
 	} else {
-		uint8_t* o = out + blk * BLOCK_BYTES;
+		uint8_t* o = out + (m * nb + b) * BLOCK_BYTES;
 		// the qs field sits at a 2-byte-aligned address: two half-word stores per lane
 		*reinterpret_cast<uint16_t*>(o + 2 + 4 * j)		= static_cast<uint16_t>(packed & 0xFFFFu);
 		*reinterpret_cast<uint16_t*>(o + 2 + 4 * j + 2) = static_cast<uint16_t>(packed >> 16);
