@@ -53,28 +53,5 @@ def build_library(verbose: bool = False, extra_flags: list[str] | None = None) -
     return LIB_PATH
 
 
-HOST_TEST_SRC = os.path.join(os.path.dirname(PKG_DIR), "tests", "cpp", "test_mul_mat_dispatch.cpp")
-HOST_TEST_BIN = os.path.join(os.path.dirname(PKG_DIR), "tests", "cpp", "test_mul_mat_dispatch")
-
-
-def build_host_tests() -> str:
-    """Compile the C++23 dispatch-surface test: a host-only translation unit (no HIP header) linked against the C ABI
-    library and the CPU checker.  Needs build_library() and oracle/ built first."""
-    root = os.path.dirname(PKG_DIR)
-    cxx = os.path.join(os.path.dirname(hipcc()), "amdclang++")
-    if not os.path.exists(cxx):
-        cxx = "/opt/rocm/bin/amdclang++"
-    oracle_dir = os.path.join(root, "oracle")
-    cmd = [
-        cxx, "-std=c++23", "-O2", "-Wall", "-Wextra", "-I", os.path.join(root, "include"), HOST_TEST_SRC, "-o", HOST_TEST_BIN,
-        "-L", PKG_DIR, "-lnihilus_q8_hip", "-L", oracle_dir, "-lq8_0_oracle",
-        f"-Wl,-rpath,$ORIGIN/../../nihilus_amd", f"-Wl,-rpath,$ORIGIN/../../oracle", "-Wl,-rpath,/opt/rocm/lib",
-    ]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"host test build failed:\n{' '.join(cmd)}\n{res.stderr}")
-    return HOST_TEST_BIN
-
-
 if __name__ == "__main__":
     print(build_library(verbose=True))
