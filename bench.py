@@ -252,7 +252,7 @@ INT8_MFMA_PEAK_TOPS = 5033.0  # MI355X published dense int8 matrix rate
 
 
 def side_workload(kind: str, steps: int, warmup: int) -> dict:
-    """One JSON line for the prefill mat-mat (BASELINE config 3: M=512, W [4096x4096] and [14336x4096]), for the
+    """One JSON line for the prefill mat-mat (the prefill benchmark configuration: M=512, W [4096x4096] and [14336x4096]), for the
     stand-alone activation quantize (M=512, K=4096) or for the token-embedding lookup (512 tokens), each against
     the roofline that bounds it."""
     import torch
@@ -332,7 +332,7 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                            "(17.8 / 62.4 MB against a 256 MB last-level cache): the GEMV -> GEMM crossover, not an HBM figure"}, "rows": rows}
 
     if kind == "llama70b":
-        # BASELINE config 5: the LLaMA-3-70B projections at batched-decode sizes; weight sets are rotated so that
+        # the LLaMA-3-70B projections at batched-decode sizes; weight sets are rotated so that
         # each launch streams its matrix from HBM (the figure is weight bytes / time, the quantize launch included)
         k70 = {"q_o": (8192, 8192), "k_v": (1024, 8192), "gate_up": (28672, 8192), "down": (8192, 28672), "lm_head": (128256, 8192)}
         rows = []
