@@ -300,12 +300,12 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
         }
 
     if kind == "crossover":
-        # M in {1, 8, 32, 128, 512} against the same two weights: where the mat-vec (HBM-bound) hands over to the
+        # M in {1, 2, 4, 8, 32, 64, 128, 512} against the same two weights: where the mat-vec (HBM-bound; M = 2, 3 still on it) hands over to the
         # weight-streaming MFMA kernel (M <= 64) and that to the MFMA tile kernel (compute-bound)
         shapes = [(4096, K), (14336, K)]
         ws = [q8_0.tile(q8_0.fill_weight_blocks(3 + i, n, k), n, k) for i, (n, k) in enumerate(shapes)]
         rows = []
-        for m in (1, 8, 32, 64, 128, 512):
+        for m in (1, 2, 4, 8, 32, 64, 128, 512):
             xm = x[:m].contiguous()
             ws_bytes = max(256, lib.nh_q8_0_mul_mat_workspace_bytes(m, K))
             wsp = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
