@@ -103,6 +103,29 @@ def test_gemv_split_k_is_deterministic_and_reusable(q8, oracle):
     assert rel_l2(first, oracle.gemv(w, xq, n, k)) <= REL_L2_TOL
 
 
+def test_split_k_back_to_back_with_changing_inputs(q8, oracle):
+    # launches that share the K-split scratch queued without a sync in between, inputs alternating: a stale partial sum of
+    # the previous launch must never be taken for a share of the current one (mat-vec, 3-row form, MFMA streaming kernel)
+    import torch
+
+    n, k = 2048, 14336
+    w = oracle.fill_weights(5, n, k)
+    wt = q8.tile(to_dev(w), n, k)
+    xs = [to_dev(oracle.fill_activations(40 + i, 8 * k).reshape(8, k)) for i in range(2)]
+    solo = []
+    for x in xs:
+        solo.append((to_host(q8.gemv_f32(wt, x[0], n, k)), to_host(q8.mul_mat(wt, x[:3], n, k)), to_host(q8.mul_mat(wt, x, n, k))))
+        torch.cuda.synchronize()
+    outs = []
+    for i in range(12):
+        x = xs[i & 1]
+        outs.append((q8.gemv_f32(wt, x[0], n, k), q8.mul_mat(wt, x[:3], n, k), q8.mul_mat(wt, x, n, k)))
+    torch.cuda.synchronize()
+    for i, got in enumerate(outs):
+        for g, want in zip(got, solo[i & 1]):
+            assert np.array_equal(to_host(g), want), i
+
+
 @pytest.mark.parametrize("k", [128, 4096, 14336, 28672, 512 * 128])
 def test_fused_quantize_stage_is_bit_exact(q8, oracle, k):
     # the quantize inside the mat-vec kernel must stage exactly the bytes the stand-alone quantizer writes
