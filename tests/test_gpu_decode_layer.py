@@ -73,3 +73,63 @@ def test_decode_layer_chain(q8, oracle, hidden, n_kv, n_ff, vocab):
     y_c = oracle.gemv(wd, a_c, hidden, n_ff) + h_c
     assert rel_l2(to_host(y), y_c) <= END_TO_END_TOL
     assert np.isfinite(to_host(y)).all()
+
+
+@pytest.mark.parametrize("m,hidden,n_kv,n_ff,vocab", [(40, 512, 128, 1536, 1000), (130, 1024, 256, 2816, 3000)])
+def test_prefill_layer_chain(q8, oracle, m, hidden, n_kv, n_ff, vocab):
+    # the same layer for M prompt tokens: get_rows -> RMS norm * weight -> quantize (one kernel, tiled output shared by q/k/v)
+    # -> mat-mats -> o -> residual -> RMS norm * weight -> quantize -> gate/up mat-mats -> SiLU * up -> quantize -> down
+    rng = np.random.default_rng(m + hidden)
+    eps = 1e-5
+
+    def sigma(k_in):
+        return 1.0 / (58.0 * np.sqrt(k_in))
+
+    emb = random_blocks(rng, vocab, hidden, 1.0 / 58.0)
+    wq, wk, wo = (random_blocks(rng, n, hidden, sigma(hidden)) for n in (hidden, n_kv, hidden))
+    wg, wu, wd = random_blocks(rng, n_ff, hidden, sigma(hidden)), random_blocks(rng, n_ff, hidden, sigma(hidden)), random_blocks(rng, hidden, n_ff, sigma(n_ff))
+    attn_norm = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    ffn_norm = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    tokens = rng.integers(0, vocab, size=m).astype(np.int32)
+    t = {name: q8.tile(to_dev(w), n, k) for name, (w, n, k) in {
+        "emb": (emb, vocab, hidden), "q": (wq, hidden, hidden), "k": (wk, n_kv, hidden), "o": (wo, hidden, hidden),
+        "g": (wg, n_ff, hidden), "u": (wu, n_ff, hidden), "d": (wd, hidden, n_ff)}.items()}
+
+    def cpu_mm(w, aq, n, k):
+        return oracle.gemm(w, aq, m, n, k, threads=4) if (k // 32) % 16 == 0 else oracle.gemm(w, aq, m, n, k)
+
+    # ---- GPU chain ----
+    x0 = q8.get_rows(t["emb"], to_dev(tokens), vocab, hidden, tiled=True)
+    a0 = q8.rms_norm_quantize(x0, to_dev(attn_norm), eps, tiled=True)
+    q = q8.gemm(t["q"], a0, m, hidden, hidden, tiled=True)
+    k_ = q8.gemm(t["k"], a0, m, n_kv, hidden, tiled=True)
+    o = q8.mul_mat(t["o"], q, hidden, hidden)  # attention stood in for by q; quantize + mat-mat in one call
+    h = x0 + o
+    a1 = q8.rms_norm_quantize(h, to_dev(ffn_norm), eps, tiled=True)
+    g = q8.gemm(t["g"], a1, m, n_ff, hidden, tiled=True)
+    u = q8.gemm(t["u"], a1, m, n_ff, hidden, tiled=True)
+    a2 = q8.silu_mul_quantize(g, u, tiled=True)
+    y = q8.gemm(t["d"], a2, m, hidden, n_ff, tiled=True) + h
+
+    # ---- stage by stage on the GPU's own inputs: quantized activations bit for bit, fp32 outputs within the contract ----
+    x0_cpu = oracle.get_rows(emb, tokens, vocab, hidden)[0]
+    assert np.array_equal(to_host(x0), x0_cpu)
+    a0_cpu = oracle.rms_norm_quantize_rows(to_host(x0), attn_norm, eps)
+    assert np.array_equal(to_host(q8.untile(a0, m, hidden)).reshape(m, -1), a0_cpu)
+    assert rel_l2(to_host(q), cpu_mm(wq, a0_cpu, hidden, hidden)) <= REL_L2_TOL
+    assert rel_l2(to_host(k_), cpu_mm(wk, a0_cpu, n_kv, hidden)) <= REL_L2_TOL
+    assert rel_l2(to_host(o), cpu_mm(wo, oracle.quantize_rows(to_host(q)), hidden, hidden)) <= REL_L2_TOL
+    a1_cpu = oracle.rms_norm_quantize_rows(to_host(h), ffn_norm, eps)
+    assert np.array_equal(to_host(q8.untile(a1, m, hidden)).reshape(m, -1), a1_cpu)
+    assert rel_l2(to_host(g), cpu_mm(wg, a1_cpu, n_ff, hidden)) <= REL_L2_TOL
+    a2_cpu = oracle.silu_mul_quantize_rows(to_host(g), to_host(u))
+    assert np.array_equal(to_host(q8.untile(a2, m, n_ff)).reshape(m, -1), a2_cpu)
+    assert rel_l2(to_host(y), cpu_mm(wd, a2_cpu, hidden, n_ff) + to_host(h)) <= REL_L2_TOL
+
+    # ---- the checker's own chain ----
+    q_c = cpu_mm(wq, oracle.rms_norm_quantize_rows(x0_cpu, attn_norm, eps), hidden, hidden)
+    h_c = x0_cpu + cpu_mm(wo, oracle.quantize_rows(q_c), hidden, hidden)
+    a1_c = oracle.rms_norm_quantize_rows(h_c, ffn_norm, eps)
+    a2_c = oracle.silu_mul_quantize_rows(cpu_mm(wg, a1_c, n_ff, hidden), cpu_mm(wu, a1_c, n_ff, hidden))
+    y_c = cpu_mm(wd, a2_c, hidden, n_ff) + h_c
+    assert rel_l2(to_host(y), y_c) <= END_TO_END_TOL
