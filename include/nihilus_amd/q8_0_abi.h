@@ -135,6 +135,9 @@ int nh_q8_0_gemv_tiled(const void* W_tiled, const void* xq_blocks, float* y, int
 /* Fused decode step: y = W . quantize(x) with the quantize done inside the mat-vec kernel (no separate launch, the
  * quantized row never travels through memory).  x: fp32 [K].  Same values as nh_q8_0_quantize + nh_q8_0_gemv_tiled. */
 int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream);
+/* The same with the residual add of the layer behind it (attn_out mul_mat -> residual add, infra/core_traits.hpp:768-772):
+ * y = W . Q(x) + residual, one fp32 add after the row's sum.  residual may be y itself (in-place accumulate). */
+int nh_q8_0_gemv_tiled_residual_f32(const void* W_tiled, const float* x, const float* residual, float* y, int64_t N, int64_t K, void* stream);
 /* The same for up to 3 weight matrices that share K and x (q/k/v, gate/up: infra/core_traits.hpp:575-594, :976-986)
  * as ONE launch: y[i] = W_tiled[i] . quantize(x), i < count.  host_* arrays are host memory, read before return. */
 int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream);

@@ -337,7 +337,7 @@ int nh_q8_0_gemv_tiled(const void* W_tiled, const void* xq_blocks, float* y, int
 }
 
 static int gemv_multi_common(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, const float* norm_weight, float eps, int64_t K,
-	void* stream) {
+	void* stream, const float* const* host_residual = nullptr) {
 	NH_REQUIRE(count >= 0 && count <= nh::GEMV_MAX_SEGMENTS, NH_ERR_ARGUMENT);
 	if (count == 0) {
 		return NH_OK;
@@ -358,6 +358,7 @@ static int gemv_multi_common(const void* const* host_W_tiled, float* const* host
 		}
 		NH_REQUIRE(host_y[i], NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(host_y[i]), NH_ERR_ALIGNMENT);
+		NH_REQUIRE(!host_residual || aligned16(host_residual[i]), NH_ERR_ALIGNMENT);
 		if (K > 0) {
 			NH_REQUIRE(host_W_tiled[i], NH_ERR_NULL_POINTER);
 			NH_REQUIRE(aligned16(host_W_tiled[i]), NH_ERR_ALIGNMENT);
@@ -370,7 +371,7 @@ static int gemv_multi_common(const void* const* host_W_tiled, float* const* host
 	NH_REQUIRE(aligned16(norm_weight), NH_ERR_ALIGNMENT);
 	NH_REQUIRE(!norm_weight || (eps >= 0.0f && eps < 1.0f), NH_ERR_ARGUMENT);
 	NH_TRY(require_device());
-	return from_hip(nh::launch_gemv_tiled_multi(host_W_tiled, host_y, host_N, static_cast<int>(count), x, true, K, as_stream(stream), norm_weight, eps));
+	return from_hip(nh::launch_gemv_tiled_multi(host_W_tiled, host_y, host_N, static_cast<int>(count), x, true, K, as_stream(stream), norm_weight, eps, host_residual));
 }
 
 int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream) {
@@ -381,6 +382,11 @@ int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* co
 	int64_t K, void* stream) {
 	NH_REQUIRE(norm_weight || K == 0 || count == 0, NH_ERR_NULL_POINTER);
 	return gemv_multi_common(host_W_tiled, host_y, host_N, count, x, norm_weight, eps, K, stream);
+}
+
+int nh_q8_0_gemv_tiled_residual_f32(const void* W_tiled, const float* x, const float* residual, float* y, int64_t N, int64_t K, void* stream) {
+	NH_REQUIRE(residual || N == 0, NH_ERR_NULL_POINTER);
+	return gemv_multi_common(&W_tiled, &y, &N, 1, x, nullptr, 0.0f, K, stream, &residual);
 }
 
 int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream) {

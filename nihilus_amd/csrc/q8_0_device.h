@@ -235,7 +235,7 @@ hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* 
 // or the fp32 activations themselves, quantized inside the kernel (x_is_f32 = true).
 constexpr int GEMV_MAX_SEGMENTS = 3;
 hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s,
-	const float* norm_w = nullptr, float norm_eps = 0.0f);
+	const float* norm_w = nullptr, float norm_eps = 0.0f, const float* const* residual = nullptr);
 // Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
 hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* norm_w, float norm_eps, const float* residual, float* y, int64_t n_ff,
 	int64_t K, int64_t n_out, hipStream_t s);

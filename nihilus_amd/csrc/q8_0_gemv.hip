@@ -177,17 +177,18 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 		}
 	}
 	const int row = strip * STRIP_ROWS + rowpart * PART_ROWS + tid;
-	float* y	  = seg.y[sidx];
+	float* y		  = seg.y[sidx];
+	const float* res  = seg.residual[sidx];
 	if (splits == 1) {
 		if (tid < PART_ROWS && row < N) {
-			y[row] = total;
+			y[row] = res ? total + res[row] : total;
 		}
 		return;
 	}
 
 	// ---- K split over several workgroups ----
 	if (tid < STRIP_ROWS) {
-		split_k_finish(tagged, epoch, gstrip, splits, split, tid, total, y, row, N, nullptr);
+		split_k_finish(tagged, epoch, gstrip, splits, split, tid, total, y, row, N, res);
 	}
 }
 
@@ -275,7 +276,7 @@ template<int RS, bool XF32> static hipError_t launch_gemv_tiled_rs(int tiles, co
 }
 
 static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, void* dump, int dump_mode, hipStream_t s,
-	const float* norm_w = nullptr, float norm_eps = 0.0f) {
+	const float* norm_w = nullptr, float norm_eps = 0.0f, const float* const* residual = nullptr) {
 	gemv_segments seg{};
 	int64_t strips = 0;
 	for (int i = 0; i < GEMV_MAX_SEGMENTS; ++i) {
@@ -283,6 +284,7 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 			seg.W[i]	= static_cast<const uint8_t*>(W[i]);
 			seg.y[i]	= y ? y[i] : nullptr;
 			seg.rows[i] = static_cast<int>(N[i]);
+			seg.residual[i] = residual ? residual[i] : nullptr;
 			strips += (N[i] + STRIP_ROWS - 1) / STRIP_ROWS;
 		}
 		seg.strip_end[i] = static_cast<int>(strips);
@@ -335,6 +337,13 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 }
 
 // y <- 0 for an empty inner dimension (a fill kernel rather than a memset node, so the call can be graph-captured)
+__global__ void copy_or_zero_f32_kernel(float* y, const float* src, int64_t n) {
+	const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+	if (i < n) {
+		y[i] = src ? src[i] : 0.0f;
+	}
+}
+
 __global__ void zero_f32_kernel(float* __restrict__ y, int64_t n) {
 	const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
 	if (i < n) {
@@ -370,16 +379,17 @@ hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* 
 	return launch_gemv_blocks_t<4>(w, x, y, sums, static_cast<int>(N), static_cast<int>(K), s);
 }
 
-hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s, const float* norm_w, float norm_eps) {
-	if (K == 0) {
+hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s, const float* norm_w, float norm_eps,
+	const float* const* residual) {
+	if (K == 0) { // empty dot products: y = residual, or 0
 		for (int i = 0; i < count; ++i) {
 			if (N[i] > 0) {
-				zero_f32_kernel<<<dim3(static_cast<unsigned>((N[i] + 255) / 256)), dim3(256), 0, s>>>(y[i], N[i]);
+				copy_or_zero_f32_kernel<<<dim3(static_cast<unsigned>((N[i] + 255) / 256)), dim3(256), 0, s>>>(y[i], residual ? residual[i] : nullptr, N[i]);
 			}
 		}
 		return hipGetLastError();
 	}
-	return launch_gemv_tiled_any(W, y, N, count, x, x_is_f32, K, nullptr, DUMP_NONE, s, x_is_f32 ? norm_w : nullptr, norm_eps);
+	return launch_gemv_tiled_any(W, y, N, count, x, x_is_f32, K, nullptr, DUMP_NONE, s, x_is_f32 ? norm_w : nullptr, norm_eps, residual);
 }
 
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w, float norm_eps) {

@@ -11,6 +11,7 @@ struct gemv_segments {
 	float* y[GEMV_MAX_SEGMENTS];
 	int rows[GEMV_MAX_SEGMENTS];
 	int strip_end[GEMV_MAX_SEGMENTS]; // running total of strips
+	const float* residual[GEMV_MAX_SEGMENTS]; // per matrix, or null: added to the finished row (one fp32 add after the sum)
 };
 
 enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };

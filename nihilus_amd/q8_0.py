@@ -170,6 +170,18 @@ def gemv_f32(w_tiled: list[torch.Tensor] | torch.Tensor, x: torch.Tensor, n: lis
     return ys[0] if single else ys
 
 
+def gemv_residual_f32(w_tiled: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, n: int, k: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """y = W . Q(x) + residual in one launch (out may be the residual tensor itself: in-place accumulate)."""
+    w_tiled, x, residual = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(x, torch.float32, "x"), _dev(residual, torch.float32, "residual")
+    if x.numel() != k or residual.numel() != n or w_tiled.numel() != tiled_bytes(n, k):
+        raise ValueError("operand sizes do not match n x k")
+    y = torch.empty(n, dtype=torch.float32, device=x.device) if out is None else _dev(out, torch.float32, "out")
+    if y.numel() != n:
+        raise ValueError("out must hold n floats")
+    _lib.check("nh_q8_0_gemv_tiled_residual_f32", _lib.lib().nh_q8_0_gemv_tiled_residual_f32(w_tiled.data_ptr(), x.data_ptr(), residual.data_ptr(), y.data_ptr(), n, k, _stream()))
+    return y
+
+
 def debug_fused_quantize(x: torch.Tensor, norm_weight: torch.Tensor | None = None, eps: float = 0.0) -> torch.Tensor:
     """The activation row exactly as the fused mat-vec stages it (after the RMS norm, if a norm weight is given), as packed blocks."""
     x = _dev(x, torch.float32, "x")

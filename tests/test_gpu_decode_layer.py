@@ -47,8 +47,8 @@ def test_decode_layer_chain(q8, oracle, hidden, n_kv, n_ff, vocab):
     ids = torch.tensor([token], dtype=torch.int32, device="cuda")
     x0 = q8.get_rows(t["emb"], ids, vocab, hidden, tiled=True).reshape(-1)
     q, k_, v = q8.gemv_f32([t["q"], t["k"], t["v"]], x0, [hidden, n_kv, n_kv], hidden, norm_weight=to_dev(attn_norm), eps=eps)
-    o = q8.gemv_f32(t["o"], q, hidden, hidden)  # the attention output is stood in for by q
-    h = x0 + o
+    h = q8.gemv_residual_f32(t["o"], q, x0, hidden, hidden)  # the attention output is stood in for by q; residual add inside the launch
+    o = h - x0
     y = q8.ffn(t["g"], t["u"], t["d"], h, n_ff, hidden, hidden, residual=h, norm_weight=to_dev(ffn_norm), eps=eps)
 
     # ---- stage by stage: the checker on the GPU's own inputs ----
@@ -57,7 +57,8 @@ def test_decode_layer_chain(q8, oracle, hidden, n_kv, n_ff, vocab):
     xq = _cpu_norm_quant(oracle, to_host(x0), attn_norm, eps)
     for got, w, n in ((q, wq, hidden), (k_, wk, n_kv), (v, wv, n_kv)):
         assert rel_l2(to_host(got), oracle.gemv(w, xq, n, hidden)) <= REL_L2_TOL
-    assert rel_l2(to_host(o), oracle.gemv(wo, oracle.quantize_rows(to_host(q))[0], hidden, hidden)) <= REL_L2_TOL
+    assert rel_l2(to_host(h), oracle.gemv(wo, oracle.quantize_rows(to_host(q))[0], hidden, hidden) + x0_cpu) <= REL_L2_TOL
+    del o
     hq = _cpu_norm_quant(oracle, to_host(h), ffn_norm, eps)
     g_gpu, u_gpu = (to_host(a) for a in q8.debug_ffn_gate_up(n_ff))
     assert rel_l2(g_gpu, oracle.gemv(wg, hq, n_ff, hidden)) <= REL_L2_TOL and rel_l2(u_gpu, oracle.gemv(wu, hq, n_ff, hidden)) <= REL_L2_TOL

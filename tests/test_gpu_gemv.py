@@ -145,6 +145,22 @@ def test_gemv_fused_f32_equals_two_step(q8, oracle, n, k):
     assert rel_l2(fused, oracle.gemv(w, xq, n, k)) <= REL_L2_TOL
 
 
+@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (100, 1024), (33, 128), (128256, 4096)])
+def test_gemv_residual(q8, oracle, n, k):
+    # y = W . Q(x) + residual: exactly one fp32 add after the row's sum, in every form of the kernel (unsplit, row parts, K split),
+    # and in place
+    w, x, xq = _inputs(oracle, n, k, seed=n + 3 * k)
+    res = oracle.fill_activations(n, n)
+    wt, xd = q8.tile(to_dev(w), n, k), to_dev(x)
+    plain = to_host(q8.gemv_f32(wt, xd, n, k))
+    got = to_host(q8.gemv_residual_f32(wt, xd, to_dev(res), n, k))
+    assert np.array_equal(got, plain + res)
+    acc = to_dev(res.copy())
+    q8.gemv_residual_f32(wt, xd, acc, n, k, out=acc)
+    assert np.array_equal(to_host(acc), got)
+    assert rel_l2(got, oracle.gemv(w, xq, n, k) + res) <= REL_L2_TOL
+
+
 def test_gemv_multi_segment(q8, oracle):
     # q/k/v-shaped and gate/up-shaped groups as one launch each; results equal the single launches bit for bit
     for ns, k in [([4096, 1024, 1024], 4096), ([14336, 14336], 4096), ([40, 33, 1], 256), ([96], 128)]:
