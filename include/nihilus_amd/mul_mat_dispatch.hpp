@@ -229,6 +229,16 @@ namespace nihilus {
 			}
 		}
 
+		// The same with the add node that follows the projection folded in (attn_out mul_mat -> residual add,
+		// infra/core_traits.hpp:768-772): output = W . quantize(activation) + residual; residual may be the output buffer.
+		static void impl_add(core_traits_type& output, const void* weight_tiled, const float* activation, const float* residual, void* stream = nullptr) {
+			amd_detail::check<config_type>(nh_q8_0_gemv_tiled_residual_f32(weight_tiled, activation, residual, output.template get_data<float>(), ne01, ne00, stream),
+				"eval_time mat-vec + residual");
+			if constexpr (config_type::synchronous) {
+				amd_detail::check<config_type>(nh_stream_sync(stream), "stream sync");
+			}
+		}
+
 		// weight: device pointer to the tiled matrix; activation: fp32 [K]; output: fp32 [N]; stream may be null
 		static void impl(core_traits_type& output, const void* weight_tiled, const float* activation, void* stream = nullptr) {
 			amd_detail::check<config_type>(nh_q8_0_gemv_tiled_f32(weight_tiled, activation, output.template get_data<float>(), ne01, ne00, stream), "eval_time mat-vec");
@@ -300,6 +310,10 @@ namespace nihilus {
 			processing_phase, mul_mat_traits_type, float, block_q8_0<half>, block_q8_0<half>>;
 		template<typename... arg_types> static void impl(arg_types&&... args) {
 			impl_type::impl(std::forward<arg_types>(args)...);
+		}
+		// eval_time only: the projection with the add node behind it folded in
+		template<typename... arg_types> static void impl_add(arg_types&&... args) {
+			impl_type::impl_add(std::forward<arg_types>(args)...);
 		}
 	};
 

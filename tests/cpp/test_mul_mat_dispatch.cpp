@@ -109,6 +109,14 @@ int main(int argc, char** argv) {
 	std::printf("eval_time        rel L2 %.3e\n", e1);
 	REQUIRE(e1 <= 1e-4);
 
+	// eval_time with the residual add folded in, in place: the buffer holds y, the same launch on top of it gives exactly 2 y
+	eval_dispatch::impl_add(op, d_tiled, static_cast<const float*>(d_x), static_cast<const float*>(d_y));
+	std::vector<float> y2(N);
+	REQUIRE(nh_memcpy_d2h(y2.data(), d_y, N * 4, nullptr) == NH_OK && nh_stream_sync(nullptr) == NH_OK);
+	for (uint64_t i = 0; i < N; ++i) {
+		REQUIRE(y2[i] == 2.0f * y[i]);
+	}
+
 	// prompt_eval_time: runtime sequence length through the dims' runtime slot
 	op.get_seq_length_dim() = M;
 	prompt_dispatch::impl(op, d_tiled, static_cast<const float*>(d_x), d_ws, ws_bytes);
