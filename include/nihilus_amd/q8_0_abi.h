@@ -170,6 +170,10 @@ int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void
  * int8 MFMA (v_mfma_i32_32x32x32_i8) per 32-quant block, fp32 scale application per block. */
 int nh_q8_0_gemm(const void* W_blocks, const void* Aq_blocks, float* C, int64_t M, int64_t N, int64_t K, void* stream);
 int nh_q8_0_gemm_tiled(const void* W_tiled, const void* Aq_tiled, float* C, int64_t M, int64_t N, int64_t K, void* stream);
+/* The tiled mat-mat with the add node behind the projection folded into its store (attn_out mul_mat -> residual add,
+ * infra/core_traits.hpp:768-772; down mul_mat -> add, :988-992): C = W . Aq + residual, one fp32 add per element after its
+ * sum.  residual: fp32 [M][N], may be C itself (in-place accumulate). */
+int nh_q8_0_gemm_tiled_residual(const void* W_tiled, const void* Aq_tiled, const float* residual, float* C, int64_t M, int64_t N, int64_t K, void* stream);
 
 /* Fused mul_mat: fp32 activations in, fp32 out -------------------------------------------------- */
 

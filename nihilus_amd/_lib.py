@@ -47,6 +47,7 @@ SIGNATURES = {
     "nh_q8_0_debug_fused_quantize": (_int, [_vp, _vp, _i64, _vp]),
     "nh_q8_0_gemm": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "nh_q8_0_gemm_tiled": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "nh_q8_0_gemm_tiled_residual": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "nh_q8_0_mul_mat_workspace_bytes": (_i64, [_i64, _i64]),
     "nh_q8_0_mul_mat": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
     "nh_q8_0_mul_mat_batch": (_int, [_vp, _i64, _vp, _i64, _vp]),

@@ -428,20 +428,20 @@ int nh_q8_0_rms_norm_quantize_tiled(const float* x, const float* norm_weight, fl
 	return rms_norm_quantize_common(x, norm_weight, eps, xq_tiled, M, K, true, stream);
 }
 
-static int gemm_common(const void* W, const void* A, float* C, int64_t M, int64_t N, int64_t K, bool tiled, void* stream) {
+static int gemm_common(const void* W, const void* A, float* C, int64_t M, int64_t N, int64_t K, bool tiled, void* stream, const float* residual = nullptr) {
 	NH_TRY(check_shape(M, N, K, tiled));
 	if (M == 0 || N == 0) {
 		return NH_OK;
 	}
 	NH_REQUIRE(M <= 65535 * 128, NH_ERR_TOO_LARGE); // grid.y
 	NH_REQUIRE(C, NH_ERR_NULL_POINTER);
-	NH_REQUIRE(aligned16(C), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(aligned16(C) && aligned16(residual), NH_ERR_ALIGNMENT);
 	if (K > 0) {
 		NH_REQUIRE(W && A, NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(W) && aligned16(A), NH_ERR_ALIGNMENT);
 	}
 	NH_TRY(require_device());
-	return from_hip(nh::launch_gemm(W, A, C, nullptr, M, N, K, tiled, as_stream(stream)));
+	return from_hip(nh::launch_gemm(W, A, C, nullptr, M, N, K, tiled, as_stream(stream), residual));
 }
 
 int nh_q8_0_gemm(const void* W_blocks, const void* Aq_blocks, float* C, int64_t M, int64_t N, int64_t K, void* stream) {
@@ -450,6 +450,11 @@ int nh_q8_0_gemm(const void* W_blocks, const void* Aq_blocks, float* C, int64_t 
 
 int nh_q8_0_gemm_tiled(const void* W_tiled, const void* Aq_tiled, float* C, int64_t M, int64_t N, int64_t K, void* stream) {
 	return gemm_common(W_tiled, Aq_tiled, C, M, N, K, true, stream);
+}
+
+int nh_q8_0_gemm_tiled_residual(const void* W_tiled, const void* Aq_tiled, const float* residual, float* C, int64_t M, int64_t N, int64_t K, void* stream) {
+	NH_REQUIRE(residual || M == 0 || N == 0, NH_ERR_NULL_POINTER);
+	return gemm_common(W_tiled, Aq_tiled, C, M, N, K, true, stream, residual);
 }
 
 int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K) {

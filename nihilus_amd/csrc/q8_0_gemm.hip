@@ -170,7 +170,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const uint8_t* __res
 //     at two waves per SIMD measured 8 % slower: with so few waves the SIMD falls back to the lone-wave issue rate
 //     whenever one of them waits.)
 template<int TM, bool DUMP, int KS = 1>
-__global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums, int M, int N,
+__global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* C, const float* R, int32_t* __restrict__ sums, int M, int N,
 	int groups) {
 	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
 	constexpr int STAGE_BYTES = DATA_BYTES + 16;
@@ -352,19 +352,20 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 			for (int e = 0; e < 16; ++e) {
 				const int m = (ms0 + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 				if (m < M && n < N) {
-					C[static_cast<int64_t>(m) * N + n] = acc[i][e];
+					const int64_t at = static_cast<int64_t>(m) * N + n;
+					C[at]			 = R ? acc[i][e] + R[at] : acc[i][e]; // R may be C: read before the write, by the same thread
 				}
 			}
 		}
 	}
 }
 
-template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int k, hipStream_t s) {
+template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s) {
 	const int groups   = k / GROUP_K;
 	const int m_strips = (m + 31) / 32, n_strips = (n + 31) / 32;
 	const dim3 grid(static_cast<unsigned>((n_strips + 3) / 4), static_cast<unsigned>((m_strips + TM - 1) / TM));
 	if (sums) {
-		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, sums, m, n, groups);
+		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, R, sums, m, n, groups);
 		return hipGetLastError();
 	}
 	// a grid that leaves SIMDs short of their four waves: K sets inside the workgroup (8 or 16 waves) make up for it
@@ -373,42 +374,42 @@ template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const u
 		ks *= 2;
 	}
 	if (ks == 4) {
-		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4>, grid, dim3(1024), 0, s, w, a, C, sums, m, n, groups);
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4>, grid, dim3(1024), 0, s, w, a, C, R, sums, m, n, groups);
 	}
 	if (ks == 2) {
-		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2>, grid, dim3(512), 0, s, w, a, C, sums, m, n, groups);
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2>, grid, dim3(512), 0, s, w, a, C, R, sums, m, n, groups);
 	}
-	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false>, grid, dim3(256), 0, s, w, a, C, sums, m, n, groups);
+	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false>, grid, dim3(256), 0, s, w, a, C, R, sums, m, n, groups);
 }
 
 // Tile choice.  One wave alone issues a VALU instruction only every ~5 cycles (two or more per SIMD reach ~2.4), so
 // the grid must give every SIMD at least two waves: 64-row workgroup tiles (half the LDS and L2 traffic per MFMA) when
 // that still leaves >= 512 workgroups, 32-row tiles otherwise.
-static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int k, hipStream_t s) {
+static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s) {
 	const int64_t ms = (m + 31) / 32;
 	// Two activation strips per wave whenever there are two: every weight tile fetched is used twice, which halves what a CU
 	// has to take in per MFMA (that intake, not the MFMA rate, bounds the one-strip form); the K sets below give back the
 	// waves the halved grid loses.
 	if (ms >= 2) {
-		return launch_gemm_tiled_t<2>(w, a, C, sums, m, n, k, s);
+		return launch_gemm_tiled_t<2>(w, a, C, R, sums, m, n, k, s);
 	}
-	return launch_gemm_tiled_t<1>(w, a, C, sums, m, n, k, s);
+	return launch_gemm_tiled_t<1>(w, a, C, R, sums, m, n, k, s);
 }
 
-__global__ void zero_c_kernel(float* __restrict__ c, int64_t n) {
+__global__ void zero_c_kernel(float* c, const float* src, int64_t n) {
 	const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
 	if (i < n) {
-		c[i] = 0.0f;
+		c[i] = src ? src[i] : 0.0f;
 	}
 }
 
-hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s) {
+hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s, const float* residual) {
 	if (M == 0 || N == 0) {
 		return hipSuccess;
 	}
-	if (K == 0) {
+	if (K == 0) { // empty dot products: C = residual, or 0
 		if (!sums) {
-			zero_c_kernel<<<dim3(static_cast<unsigned>((M * N + 255) / 256)), dim3(256), 0, s>>>(C, M * N);
+			zero_c_kernel<<<dim3(static_cast<unsigned>((M * N + 255) / 256)), dim3(256), 0, s>>>(C, residual, M * N);
 		}
 		return hipGetLastError();
 	}
@@ -423,9 +424,9 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 		// waves of a workgroup, the weights coming from cache after the first group.
 		const int64_t tile_workgroups = ((N + 127) / 128) * ((M + 31) / 32);
 		if (M <= GEMM_SKINNY_MAX_M || tile_workgroups <= 256) {
-			return launch_gemm_skinny(W, Aq, C, sums, M, N, K, s);
+			return launch_gemm_skinny(W, Aq, C, sums, M, N, K, s, residual);
 		}
-		return launch_gemm_tiled(w, a, C, sums, m, n, k, s);
+		return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s);
 	} else {
 		if (sums) {
 			gemm_kernel<false, true><<<grid, dim3(GEMM_THREADS), 0, s>>>(w, a, C, sums, m, n, k);

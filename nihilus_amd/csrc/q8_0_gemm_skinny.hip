@@ -26,7 +26,7 @@ __device__ __forceinline__ v2u scale_slot(v2u four, int t) {
 }
 
 template<int MS, bool DUMP, int GC>
-__global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* __restrict__ C, int32_t* __restrict__ sums,
+__global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* C, const float* R, int32_t* __restrict__ sums,
 	float* __restrict__ partials, unsigned* __restrict__ counters, int M, int N, int groups, int split_shift) {
 	__shared__ float red[SK_WAVES / 2][MS][16][64];
 	__shared__ int last_flag;
@@ -179,7 +179,8 @@ __global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kerne
 				for (int e = 0; e < 16; ++e) {
 					const int m = (mg * MS + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 					if (m < M) {
-						C[static_cast<int64_t>(m) * N + n] = acc[i][e];
+						const int64_t at = static_cast<int64_t>(m) * N + n;
+						C[at]			 = R ? acc[i][e] + R[at] : acc[i][e]; // R may be C: read before the write, by the same thread
 					}
 				}
 			}
@@ -242,7 +243,8 @@ __global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kerne
 			for (int e = 0; e < 16; ++e) {
 				const int m = (mg * MS + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
 				if (m < M) {
-					C[static_cast<int64_t>(m) * N + n] = sum[i][e];
+					const int64_t at = static_cast<int64_t>(m) * N + n;
+					C[at]			 = R ? sum[i][e] + R[at] : sum[i][e];
 				}
 			}
 		}
@@ -289,7 +291,7 @@ static hipError_t get_skinny_scratch(skinny_scratch* out) {
 	return hipSuccess;
 }
 
-template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8_t* a, float* C, int32_t* sums, int m, int n, int groups, hipStream_t s) {
+template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int groups, hipStream_t s) {
 	const int strips   = (n + STRIP_ROWS - 1) / STRIP_ROWS;
 	const int m_groups = ((m + STRIP_ROWS - 1) / STRIP_ROWS + MS - 1) / MS;
 	const int units	   = strips * m_groups;
@@ -317,13 +319,13 @@ template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8
 	}
 	const dim3 grid(static_cast<unsigned>(strips * splits), static_cast<unsigned>(m_groups)), block(SK_WAVES * 64);
 	if (sums) {
-		gemm_skinny_kernel<MS, true, 1><<<grid, block, 0, s>>>(w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift);
+		gemm_skinny_kernel<MS, true, 1><<<grid, block, 0, s>>>(w, a, C, R, sums, sc.partials, sc.counters, m, n, groups, shift);
 		return hipGetLastError();
 	}
-	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, 2>, grid, block, 0, s, w, a, C, sums, sc.partials, sc.counters, m, n, groups, shift);
+	return launch_kernel(KIND_GEMM, gemm_skinny_kernel<MS, false, 2>, grid, block, 0, s, w, a, C, R, sums, sc.partials, sc.counters, m, n, groups, shift);
 }
 
-hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual) {
 	const uint8_t* w = static_cast<const uint8_t*>(W);
 	const uint8_t* a = static_cast<const uint8_t*>(Aq);
 	const int groups = static_cast<int>(K / GROUP_K);
@@ -331,9 +333,9 @@ hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* 
 	// without them: 64 rows against 128 weight strips are better off as 256 workgroups of one strip each.
 	const int64_t strips = (N + STRIP_ROWS - 1) / STRIP_ROWS, m_strips = (M + STRIP_ROWS - 1) / STRIP_ROWS;
 	if (m_strips <= 1 || strips * ((m_strips + 1) / 2) < 256) {
-		return launch_skinny_t<1>(w, a, C, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
+		return launch_skinny_t<1>(w, a, C, residual, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
 	}
-	return launch_skinny_t<2>(w, a, C, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
+	return launch_skinny_t<2>(w, a, C, residual, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
 }
 
 } // namespace nh

@@ -222,6 +222,18 @@ def gemm(w: torch.Tensor, aq: torch.Tensor, m: int, n: int, k: int, tiled: bool)
     return c
 
 
+def gemm_residual(w_tiled: torch.Tensor, aq_tiled: torch.Tensor, residual: torch.Tensor, m: int, n: int, k: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """C = W . Aq + residual on tiled operands in one launch (out may be the residual tensor itself: in-place accumulate)."""
+    w, aq, residual = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(aq_tiled, torch.uint8, "aq_tiled"), _dev(residual, torch.float32, "residual")
+    if w.numel() != tiled_bytes(n, k) or aq.numel() != tiled_bytes(m, k) or residual.numel() != m * n:
+        raise ValueError("operand sizes do not match m x n x k")
+    c = torch.empty((m, n), dtype=torch.float32, device=w.device) if out is None else _dev(out, torch.float32, "out")
+    if c.numel() != m * n:
+        raise ValueError("out must hold m x n floats")
+    _lib.check("nh_q8_0_gemm_tiled_residual", _lib.lib().nh_q8_0_gemm_tiled_residual(w.data_ptr(), aq.data_ptr(), residual.data_ptr(), c.data_ptr(), m, n, k, _stream()))
+    return c
+
+
 def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: torch.Tensor | None = None) -> torch.Tensor:
     """fp32 activations [M, K] x tiled Q8_0 weight [N, K] -> fp32 [M, N]: quantize + GEMV/GEMM."""
     w_tiled, x = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(x, torch.float32, "x")

@@ -110,7 +110,7 @@ def test_prefill_layer_chain(q8, oracle, m, hidden, n_kv, n_ff, vocab):
     g = q8.gemm(t["g"], a1, m, n_ff, hidden, tiled=True)
     u = q8.gemm(t["u"], a1, m, n_ff, hidden, tiled=True)
     a2 = q8.silu_mul_quantize(g, u, tiled=True)
-    y = q8.gemm(t["d"], a2, m, hidden, n_ff, tiled=True) + h
+    y = q8.gemm_residual(t["d"], a2, h, m, hidden, n_ff)  # the down projection with the layer's second residual add in its store
 
     # ---- stage by stage on the GPU's own inputs: quantized activations bit for bit, fp32 outputs within the contract ----
     x0_cpu = oracle.get_rows(emb, tokens, vocab, hidden)[0]

@@ -40,6 +40,21 @@ def test_gemm_block_sums_exact(q8, oracle, m, n, k):
         assert np.array_equal(got_t, got)
 
 
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (40, 512, 1024), (16, 2048, 14336), (64, 4096, 4096), (130, 257, 512), (8, 96, 256), (256, 14336, 4096)])
+def test_gemm_residual(q8, oracle, m, n, k):
+    # C = W . Aq + residual: exactly one fp32 add per element after its sum, in the MFMA tile kernel (one and two row strips, K
+    # sets) and in the streaming kernel (one and two row strips, K split over workgroups), also in place
+    w, x, aq = _inputs(oracle, m, n, k, seed=m * 7 + n)
+    res = oracle.fill_activations(m + n, m * n).reshape(m, n)
+    wt, at = q8.tile(to_dev(w), n, k), q8.tile(to_dev(aq.reshape(-1)), m, k)
+    plain = to_host(q8.gemm(wt, at, m, n, k, tiled=True))
+    got = to_host(q8.gemm_residual(wt, at, to_dev(res), m, n, k))
+    assert np.array_equal(got, plain + res)
+    acc = to_dev(res.copy())
+    q8.gemm_residual(wt, at, acc, m, n, k, out=acc)
+    assert np.array_equal(to_host(acc), got)
+
+
 def test_gemm_equals_gemvs(q8, oracle):
     # the mat-mat must be M independent mat-vecs on the same quantized rows
     m, n, k = 16, 512, 1024
