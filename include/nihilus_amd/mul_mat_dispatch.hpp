@@ -274,6 +274,21 @@ namespace nihilus {
 				amd_detail::check<config_type>(nh_stream_sync(stream), "stream sync");
 			}
 		}
+			// The same with the add node behind the projection folded in (infra/core_traits.hpp:768-772, :988-992): output = mul_mat + residual,
+		// residual fp32 [sequence_length][N], may be the output buffer.
+		static void impl_add(core_traits_type& output, const void* weight_tiled, const float* activation, const float* residual, void* workspace, int64_t workspace_size,
+			void* stream = nullptr) {
+			const uint64_t sequence_length = output.get_seq_length_dim();
+			if (sequence_length == 0) {
+				return;
+			}
+			amd_detail::check<config_type>(nh_q8_0_mul_mat_residual(weight_tiled, activation, residual, output.template get_data<float>(), static_cast<int64_t>(sequence_length), ne01,
+											   ne00, workspace, workspace_size, stream),
+				"prompt_eval_time mat-mat + residual");
+			if constexpr (config_type::synchronous) {
+				amd_detail::check<config_type>(nh_stream_sync(stream), "stream sync");
+			}
+		}
 	};
 
 	// get_rows (token embeddings), both phases: out[t][:] = dequantized row ids[t] of the embedding table.  The table
@@ -311,7 +326,7 @@ namespace nihilus {
 		template<typename... arg_types> static void impl(arg_types&&... args) {
 			impl_type::impl(std::forward<arg_types>(args)...);
 		}
-		// eval_time only: the projection with the add node behind it folded in
+		// the projection with the add node behind it folded in
 		template<typename... arg_types> static void impl_add(arg_types&&... args) {
 			impl_type::impl_add(std::forward<arg_types>(args)...);
 		}

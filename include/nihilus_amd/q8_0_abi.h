@@ -183,6 +183,10 @@ int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K);
 /* quantize(x) then GEMV (M == 1; M = 2, 3: the same kernel with one dot product per row) or GEMM (M > 3) against a tiled weight: the whole
  * rms_norm-output -> projection step of core_traits.hpp:575-594 / :976-989 as one call. */
 int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
+/* The same with the add node behind the projection folded in: y = mul_mat(W, x) + residual (fp32 [M][N], may be y itself),
+ * for any M (the attn_out and down projections of core_traits.hpp:768-772, :988-992 in either phase). */
+int nh_q8_0_mul_mat_residual(const void* W_tiled, const float* x, const float* residual, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+	void* stream);
 
 /* One entry of a batch: y[M][N] = mul_mat(W_tiled [N x K], x fp32 [M][K]).  reuse_quantized_x != 0 lets the runner
  * skip the quantize when the previous entry quantized the same x pointer with the same M and K (q/k/v share the

@@ -467,7 +467,7 @@ int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K) {
 	return (nh_q8_0_tiled_bytes(M, K) + 255) / 256 * 256;
 }
 
-int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
+static int mul_mat_common(const void* W_tiled, const float* x, const float* residual, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
 	NH_TRY(check_shape(M, N, K, true));
 	if (M == 0 || N == 0) {
 		return NH_OK;
@@ -478,17 +478,27 @@ int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, in
 		NH_REQUIRE(x && (workspace || need == 0), NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(workspace) && aligned16(x), NH_ERR_ALIGNMENT);
 	}
-	if (M == 1) {
-		return nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream); // quantize fused into the mat-vec: the workspace stays unused
+	if (M == 1) { // quantize fused into the mat-vec: the workspace stays unused
+		return residual ? nh_q8_0_gemv_tiled_residual_f32(W_tiled, x, residual, y, N, K, stream) : nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream);
 	}
 	if (M <= nh::GEMV_ROWS_MAX && K > 0) { // a few rows: the same streaming kernel with M dot products per weight tile
 		NH_REQUIRE(W_tiled && y, NH_ERR_NULL_POINTER);
-		NH_REQUIRE(aligned16(W_tiled) && aligned16(y), NH_ERR_ALIGNMENT);
+		NH_REQUIRE(aligned16(W_tiled) && aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
 		NH_TRY(require_device());
-		return from_hip(nh::launch_gemv_rows(W_tiled, x, y, M, N, K, as_stream(stream)));
+		return from_hip(nh::launch_gemv_rows(W_tiled, x, y, M, N, K, as_stream(stream), residual));
 	}
 	NH_TRY(nh_q8_0_quantize_tiled(x, workspace, M, K, stream));
-	return nh_q8_0_gemm_tiled(W_tiled, workspace, y, M, N, K, stream);
+	return residual ? nh_q8_0_gemm_tiled_residual(W_tiled, workspace, residual, y, M, N, K, stream) : nh_q8_0_gemm_tiled(W_tiled, workspace, y, M, N, K, stream);
+}
+
+int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
+	return mul_mat_common(W_tiled, x, nullptr, y, M, N, K, workspace, workspace_bytes, stream);
+}
+
+int nh_q8_0_mul_mat_residual(const void* W_tiled, const float* x, const float* residual, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+	void* stream) {
+	NH_REQUIRE(residual || M == 0 || N == 0, NH_ERR_NULL_POINTER);
+	return mul_mat_common(W_tiled, x, residual, y, M, N, K, workspace, workspace_bytes, stream);
 }
 
 int nh_q8_0_debug_block_sums(const void* W, const void* Aq, int32_t* sums, int64_t M, int64_t N, int64_t K, int path, void* stream) {

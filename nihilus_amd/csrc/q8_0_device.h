@@ -244,7 +244,7 @@ hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_
 // 2 <= M <= GEMV_ROWS_MAX fp32 activation rows against one tiled weight matrix: the streaming mat-vec with M dot products per
 // weight tile, quantize included (q8_0_gemv_rows.hip).  y is [M][N].
 constexpr int64_t GEMV_ROWS_MAX = 3;
-hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s);
+hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual = nullptr);
 // residual (tiled operands only, or null): C = W . Aq + residual, one fp32 add per element after its sum; may be C itself
 hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s, const float* residual = nullptr);
 // Tiled operands, M <= GEMM_SKINNY_MAX_M (or a tile-kernel grid of at most one workgroup per CU): the streaming MFMA kernel

@@ -112,7 +112,7 @@ __device__ __forceinline__ void gemv_rows_chunk(const uint8_t* __restrict__ w_st
 // TILES <= 2 groups per wave and chunk: MR slices of fp32 activations sit in registers next to the weight tiles (two rows fit
 // in 64 registers = two workgroups per CU; three take 65 and run as one, which measured faster than spilling to stay at two).
 template<int TILES, int MR, bool LOOP>
-__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_rows_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, uint64_t* __restrict__ tagged, unsigned epoch,
+__global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_rows_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* y, const float* residual, uint64_t* __restrict__ tagged, unsigned epoch,
 	int N, int groups, int split_shift) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][MR][TILES * GROUP_K]; // each wave's quantized slices, block jj of row m at 32*jj
 	__shared__ float xs_d[GEMV_WAVES][MR][TILES * GROUP_BLOCKS];
@@ -158,33 +158,34 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_rows_kernel(const uint8_
 		total += red[m][w][l] + red[m][w][32 + l];
 	}
 	const int row = strip * STRIP_ROWS + l;
-	float* ym	  = y + static_cast<int64_t>(m) * N;
+	float* ym		= y + static_cast<int64_t>(m) * N;
+	const float* rm = residual ? residual + static_cast<int64_t>(m) * N : nullptr; // may be ym: read before the write, by the same thread
 	if (splits == 1) {
 		if (row < N) {
-			ym[row] = total;
+			ym[row] = rm ? total + rm[row] : total;
 		}
 		return;
 	}
-	split_k_finish(tagged, epoch, strip * MR + m, splits, split, l, total, ym, row, N, nullptr);
+	split_k_finish(tagged, epoch, strip * MR + m, splits, split, l, total, ym, row, N, rm);
 }
 
-template<int TILES, int MR, bool LOOP> static hipError_t launch_rows_n(const gemv_plan& p, const uint8_t* W, const float* x, float* y, int N, const gemv_scratch& sc, hipStream_t s) {
+template<int TILES, int MR, bool LOOP> static hipError_t launch_rows_n(const gemv_plan& p, const uint8_t* W, const float* x, float* y, const float* r, int N, const gemv_scratch& sc, hipStream_t s) {
 	const dim3 grid(static_cast<unsigned>(p.strips * p.splits)), block(GEMV_WAVES * 64);
 	int shift = 0;
 	while ((1 << shift) < p.splits) {
 		++shift;
 	}
-	return launch_kernel(KIND_GEMV, gemv_rows_kernel<TILES, MR, LOOP>, grid, block, 0, s, W, x, y, sc.tagged, sc.epoch, N, p.groups, shift);
+	return launch_kernel(KIND_GEMV, gemv_rows_kernel<TILES, MR, LOOP>, grid, block, 0, s, W, x, y, r, sc.tagged, sc.epoch, N, p.groups, shift);
 }
 
-template<int MR> static hipError_t launch_rows_m(const gemv_plan& p, const uint8_t* W, const float* x, float* y, int N, const gemv_scratch& sc, hipStream_t s) {
+template<int MR> static hipError_t launch_rows_m(const gemv_plan& p, const uint8_t* W, const float* x, float* y, const float* r, int N, const gemv_scratch& sc, hipStream_t s) {
 	if (p.tiles > 2) {
-		return launch_rows_n<2, MR, true>(p, W, x, y, N, sc, s);
+		return launch_rows_n<2, MR, true>(p, W, x, y, r, N, sc, s);
 	}
-	return p.tiles <= 1 ? launch_rows_n<1, MR, false>(p, W, x, y, N, sc, s) : launch_rows_n<2, MR, false>(p, W, x, y, N, sc, s);
+	return p.tiles <= 1 ? launch_rows_n<1, MR, false>(p, W, x, y, r, N, sc, s) : launch_rows_n<2, MR, false>(p, W, x, y, r, N, sc, s);
 }
 
-hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s) {
+hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual) {
 	const int64_t strips = (N + STRIP_ROWS - 1) / STRIP_ROWS;
 	if (strips == 0 || M < 2 || M > GEMV_ROWS_MAX) {
 		return M < 2 || M > GEMV_ROWS_MAX ? hipErrorInvalidValue : hipSuccess;
@@ -211,9 +212,9 @@ hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, 
 	const int n		 = static_cast<int>(N);
 	switch (M) {
 		case 2:
-			return launch_rows_m<2>(p, w, x, y, n, sc, s);
+			return launch_rows_m<2>(p, w, x, y, residual, n, sc, s);
 		default:
-			return launch_rows_m<3>(p, w, x, y, n, sc, s);
+			return launch_rows_m<3>(p, w, x, y, residual, n, sc, s);
 	}
 }
 

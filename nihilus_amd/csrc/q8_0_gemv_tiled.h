@@ -336,6 +336,14 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 __device__ __forceinline__ void split_k_finish(uint64_t* __restrict__ tagged, unsigned epoch, int gstrip, int splits, int split, int lane, float total, float* __restrict__ y, int row,
 	int N, const float* __restrict__ residual) {
 	uint64_t* mine = tagged + static_cast<int64_t>(gstrip) * splits * STRIP_ROWS + lane;
+	// The residual may be y itself, and more than one workgroup may store the row: each takes its copy of the residual before
+	// it publishes its own share.  Nobody can have stored the row by then (that takes every share, this one included), so all
+	// of them add the same value, whoever stores first.
+	float res = 0.0f;
+	if (residual && row < N) {
+		res = residual[row];
+	}
+	asm volatile("" : "+v"(res)::"memory"); // the value is in a register (the load has returned) before the share goes out
 	__hip_atomic_store(&mine[split * STRIP_ROWS], (static_cast<uint64_t>(epoch) << 32) | __float_as_uint(total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 	wait_stores_acknowledged();
 	bool all  = true;
@@ -355,7 +363,7 @@ __device__ __forceinline__ void split_k_finish(uint64_t* __restrict__ tagged, un
 		}
 	}
 	if (all && row < N) {
-		y[row] = residual ? sum + residual[row] : sum;
+		y[row] = residual ? sum + res : sum;
 	}
 }
 

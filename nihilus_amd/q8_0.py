@@ -234,8 +234,8 @@ def gemm_residual(w_tiled: torch.Tensor, aq_tiled: torch.Tensor, residual: torch
     return c
 
 
-def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: torch.Tensor | None = None) -> torch.Tensor:
-    """fp32 activations [M, K] x tiled Q8_0 weight [N, K] -> fp32 [M, N]: quantize + GEMV/GEMM."""
+def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: torch.Tensor | None = None, residual: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 activations [M, K] x tiled Q8_0 weight [N, K] -> fp32 [M, N]: quantize + GEMV/GEMM (+ residual [M, N] if given)."""
     w_tiled, x = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(x, torch.float32, "x")
     x2 = x.reshape(1, -1) if x.dim() == 1 else x
     m = x2.shape[0]
@@ -246,6 +246,13 @@ def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: t
     if workspace is None:
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
     y = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    if residual is not None:
+        residual = _dev(residual, torch.float32, "residual")
+        if residual.numel() != m * n:
+            raise ValueError("residual must hold m x n floats")
+        _lib.check("nh_q8_0_mul_mat_residual", _lib.lib().nh_q8_0_mul_mat_residual(w_tiled.data_ptr(), x2.data_ptr(), residual.data_ptr(), y.data_ptr(), m, n, k, workspace.data_ptr(),
+                                                                             workspace.numel(), _stream()))
+        return y
     _lib.check("nh_q8_0_mul_mat", _lib.lib().nh_q8_0_mul_mat(w_tiled.data_ptr(), x2.data_ptr(), y.data_ptr(), m, n, k, workspace.data_ptr(), workspace.numel(), _stream()))
     return y
 

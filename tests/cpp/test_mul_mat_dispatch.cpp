@@ -126,6 +126,14 @@ int main(int argc, char** argv) {
 	std::printf("prompt_eval_time rel L2 %.3e  (M = %lld)\n", e2, static_cast<long long>(M));
 	REQUIRE(e2 <= 1e-4);
 
+	// the same with the residual add folded in, in place on the buffer that holds C: exactly 2 C
+	prompt_dispatch::impl_add(op, d_tiled, static_cast<const float*>(d_x), static_cast<const float*>(d_y), d_ws, ws_bytes);
+	std::vector<float> c2(M * N);
+	REQUIRE(nh_memcpy_d2h(c2.data(), d_y, M * N * 4, nullptr) == NH_OK && nh_stream_sync(nullptr) == NH_OK);
+	for (uint64_t i = 0; i < M * N; ++i) {
+		REQUIRE(c2[i] == 2.0f * c[i]);
+	}
+
 	// empty sequence: nothing is launched, nothing changes
 	op.get_seq_length_dim() = 0;
 	prompt_dispatch::impl(op, d_tiled, static_cast<const float*>(d_x), d_ws, ws_bytes);

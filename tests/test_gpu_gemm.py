@@ -55,6 +55,20 @@ def test_gemm_residual(q8, oracle, m, n, k):
     assert np.array_equal(to_host(acc), got)
 
 
+def test_mul_mat_residual_every_row_count(q8, oracle):
+    # y = mul_mat(W, x) + residual through one entry point whatever M picks underneath: mat-vec, 2- and 3-row form, streaming and
+    # tile mat-mat; one fp32 add per element after its sum
+    n, k = 384, 1024
+    w = oracle.fill_weights(3, n, k)
+    wt = q8.tile(to_dev(w), n, k)
+    for m in (1, 2, 3, 4, 40, 200):
+        x = to_dev(oracle.fill_activations(m, m * k).reshape(m, k))
+        res = oracle.fill_activations(100 + m, m * n).reshape(m, n)
+        plain = to_host(q8.mul_mat(wt, x, n, k)).reshape(m, n)
+        got = to_host(q8.mul_mat(wt, x, n, k, residual=to_dev(res))).reshape(m, n)
+        assert np.array_equal(got, plain + res), m
+
+
 def test_gemm_equals_gemvs(q8, oracle):
     # the mat-mat must be M independent mat-vecs on the same quantized rows
     m, n, k = 16, 512, 1024
