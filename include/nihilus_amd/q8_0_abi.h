@@ -70,6 +70,11 @@ int nh_memcpy_d2h(void* host_dst, const void* src_dev, int64_t bytes, void* stre
 int nh_memset(void* dst_dev, int value, int64_t bytes, void* stream);
 /* Blocks until the stream has drained: the cudaDeviceSynchronize after each launch in cuda/cuda_12.hpp:679. */
 int nh_stream_sync(void* stream);
+/* Allocates, for the current device, the two internal scratch buffers that K-split launches hand partial sums through
+ * (about 2.6 MiB and 16 MiB; otherwise made by the first launch that needs one).  After it no launch entry point of this library
+ * allocates device memory: call it once per device before capturing launches into a HIP graph or entering a serving loop.
+ * No counterpart in the reference, whose kernels never allocate (infra/model.hpp:241 owns the arena). */
+int nh_q8_0_prepare(void);
 
 /* Activation quantize -------------------------------------------------------------------------- */
 

@@ -384,6 +384,12 @@ int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* co
 	return gemv_multi_common(host_W_tiled, host_y, host_N, count, x, norm_weight, eps, K, stream);
 }
 
+int nh_q8_0_prepare(void) {
+	NH_TRY(require_device());
+	const hipError_t e = nh::prepare_gemv_scratch();
+	return from_hip(e != hipSuccess ? e : nh::prepare_gemm_scratch());
+}
+
 int nh_q8_0_gemv_tiled_residual_f32(const void* W_tiled, const float* x, const float* residual, float* y, int64_t N, int64_t K, void* stream) {
 	NH_REQUIRE(residual || N == 0, NH_ERR_NULL_POINTER);
 	return gemv_multi_common(&W_tiled, &y, &N, 1, x, nullptr, 0.0f, K, stream, &residual);

@@ -202,6 +202,18 @@ __device__ __forceinline__ void wave_k_range(int groups, int split_shift, int sp
 	g1 = g0 + w_q + (wave < w_r ? 1 : 0);
 }
 
+// True while `s` is being captured into a HIP graph.  A captured launch is replayed with the arguments it was recorded with,
+// so nothing a replay-unsafe protocol hands to the kernel per launch (the epoch of the K-split hand-off and of the one-launch
+// FFN's published blocks) would change between replays: launchers pick forms without such state for a capturing stream.
+inline bool stream_is_capturing(hipStream_t s) {
+	hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+	if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+		(void)hipGetLastError();
+		return false;
+	}
+	return st != hipStreamCaptureStatusNone;
+}
+
 // When timing is on for `kind` and the event pool has room, hands out an event pair for the next launch.
 bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop);
 
@@ -250,6 +262,9 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 // Tiled operands, M <= GEMM_SKINNY_MAX_M (or a tile-kernel grid of at most one workgroup per CU): the streaming MFMA kernel
 // of batched decode (q8_0_gemm_skinny.hip), which walks larger M in groups of 64 rows.
 constexpr int64_t GEMM_SKINNY_MAX_M = 64;
+// Make this device's K-split scratch buffers now (otherwise: on the first launch that needs one).
+hipError_t prepare_gemv_scratch();
+hipError_t prepare_gemm_scratch();
 hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual = nullptr);
 
 } // namespace nh

@@ -191,6 +191,27 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	if (e != hipSuccess) {
 		return e;
 	}
+	if (stream_is_capturing(s)) {
+		// A replayed graph runs the kernel with the epoch it was captured with, so the published blocks of one replay would
+		// pass for those of the next.  Under capture the step is three launches instead, none of which keeps state between
+		// launches: gate/up mat-vecs (norm inside) -> SiLU * up -> quantize -> down mat-vec (+ residual).  The gate / up
+		// values land where the one-launch form leaves its inspection copies.
+		const void* w2[2] = { w_gate, w_up };
+		float* y2[2]	  = { sc.gate_up, sc.gate_up + FFN_MAX_HIDDEN };
+		const int64_t n2[2] = { n_ff, n_ff };
+		hipError_t e2		= launch_gemv_tiled_multi(w2, y2, n2, 2, x, true, K, s, norm_w, norm_eps);
+		if (e2 != hipSuccess) {
+			return e2;
+		}
+		e2 = launch_silu_mul_quantize(sc.gate_up, sc.gate_up + FFN_MAX_HIDDEN, sc.act_blocks, 1, n_ff, false, s);
+		if (e2 != hipSuccess) {
+			return e2;
+		}
+		const void* w1[1]		= { w_down };
+		float* y1[1]			= { y };
+		const float* r1[1]		= { residual };
+		return launch_gemv_tiled_multi(w1, y1, &n_out, 1, sc.act_blocks, false, n_ff, s, nullptr, 0.0f, r1);
+	}
 	// the down projection: K over as many workgroups per strip as it takes for a wave to own at most 4 groups
 	const int strips_c = static_cast<int>((n_out + STRIP_ROWS - 1) / STRIP_ROWS);
 	const int groups_c = static_cast<int>(n_ff / GROUP_K);

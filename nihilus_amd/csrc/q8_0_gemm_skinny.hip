@@ -291,6 +291,11 @@ static hipError_t get_skinny_scratch(skinny_scratch* out) {
 	return hipSuccess;
 }
 
+hipError_t prepare_gemm_scratch() {
+	skinny_scratch sc;
+	return get_skinny_scratch(&sc);
+}
+
 template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int groups, hipStream_t s) {
 	const int strips   = (n + STRIP_ROWS - 1) / STRIP_ROWS;
 	const int m_groups = ((m + STRIP_ROWS - 1) / STRIP_ROWS + MS - 1) / MS;

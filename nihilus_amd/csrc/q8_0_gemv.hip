@@ -207,7 +207,7 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	gemv_scratch& sc = per_device[dev];
 	if (!sc.tagged) {
 		void* p			   = nullptr;
-		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * (8 + 1 + 1) * 4;
+		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * (8 + 1 + 1) * 4 + (FFN_MAX_HIDDEN / QK) * BLOCK_BYTES;
 		e				   = hipMalloc(&p, bytes);
 		if (e != hipSuccess) {
 			return e;
@@ -222,6 +222,7 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 		sc.act_q	= reinterpret_cast<uint32_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
 		sc.act_d	= reinterpret_cast<float*>(sc.act_q + (FFN_MAX_HIDDEN / STRIP_ROWS) * 8);
 		sc.flags	= reinterpret_cast<unsigned*>(sc.act_d + FFN_MAX_HIDDEN / STRIP_ROWS);
+		sc.act_blocks = reinterpret_cast<uint8_t*>(sc.flags + FFN_MAX_HIDDEN / STRIP_ROWS); // 16-byte aligned: every part before it is a multiple of 16 bytes
 	}
 	if (next_epoch) {
 		++sc.epoch; // flags start at zero and the first epoch handed out is 1
@@ -231,6 +232,11 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	}
 	*out = sc;
 	return hipSuccess;
+}
+
+hipError_t prepare_gemv_scratch() {
+	gemv_scratch sc;
+	return get_gemv_scratch(&sc);
 }
 
 template<int TILES, bool XF32, bool LOOP, bool NORM, int RS = 1> static hipError_t launch_gemv_tiled_n(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
@@ -292,7 +298,11 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 	if (strips == 0) {
 		return hipSuccess;
 	}
-	const gemv_plan p = plan_gemv(strips, K);
+	gemv_plan p = plan_gemv(strips, K);
+	if (p.splits > 1 && stream_is_capturing(s)) { // replay-safe form: every workgroup walks all of K (slower on long-K shapes, no per-launch state)
+		p.splits = 1;
+		p.tiles	 = (p.groups + GEMV_WAVES - 1) / GEMV_WAVES;
+	}
 	gemv_scratch sc;
 	if (p.splits > 1) {
 		const hipError_t e = get_gemv_scratch(&sc, true);

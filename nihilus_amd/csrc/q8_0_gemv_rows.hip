@@ -200,6 +200,9 @@ hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, 
 	while (tiles_for(p.splits) > 2 && strips * M * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
 		p.splits *= 2;
 	}
+	if (p.splits > 1 && stream_is_capturing(s)) { // replay-safe form: no K split, chunked walk instead
+		p.splits = 1;
+	}
 	p.tiles = tiles_for(p.splits);
 	gemv_scratch sc;
 	if (p.splits > 1) {

@@ -379,6 +379,7 @@ struct gemv_scratch {
 	uint32_t* act_q	   = nullptr; // [FFN_MAX_HIDDEN / 32][8]: the quantized activation of the down projection, 8 dwords per block
 	float* act_d	   = nullptr; // [FFN_MAX_HIDDEN / 32]: its scales (the fp16-rounded value, widened)
 	unsigned* flags	   = nullptr; // [FFN_MAX_HIDDEN / 32]: the epoch of the launch that last published the block
+	uint8_t* act_blocks = nullptr; // [FFN_MAX_HIDDEN / 32] packed 34-byte blocks: the activation of the three-launch form used under graph capture
 	unsigned epoch	   = 0; // with next_epoch = true: a value no earlier launch on this device has used
 };
 hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch = false);

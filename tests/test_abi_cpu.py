@@ -87,6 +87,7 @@ def test_fails_loudly_without_a_gpu():
     lib = _lib.lib()
     p = C.c_void_p()
     assert lib.nh_malloc(C.byref(p), 1024) == -4  # no device: an error, never a silent CPU path
+    assert lib.nh_q8_0_prepare() == -4
     assert lib.nh_q8_0_quantize(0x1000, 0x2000, 1, 32, None) == -4
     with pytest.raises(_lib.Q8Error):
         _lib.check("nh_q8_0_quantize", lib.nh_q8_0_quantize(0x1000, 0x2000, 1, 32, None))

@@ -1,0 +1,62 @@
+"""GPU: launches captured into a HIP graph and replayed.
+
+A replay runs every kernel with the arguments it was recorded with.  The K-split hand-off of the mat-vec and the published
+blocks of the one-launch FFN are tagged with a per-launch epoch that the host hands to the kernel, which a replay cannot
+renew: the launchers therefore pick forms without per-launch state for a capturing stream (no K split in the mat-vec and its
+2- and 3-row form, three launches for the FFN; the MFMA streaming kernel's arrival counters reset themselves).  The test
+captures one of each on long-K shapes, where the eager forms do split, replays the graph several times with new inputs and
+with eager launches of the same entry points in between, and checks every replay against the eager results.
+"""
+import numpy as np
+import pytest
+
+from helpers import REL_L2_TOL, random_blocks, rel_l2, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def test_captured_launches_replay_with_new_inputs(q8, oracle):
+    import torch
+
+    from nihilus_amd import _lib
+
+    _lib.check("nh_q8_0_prepare", _lib.lib().nh_q8_0_prepare())  # every internal buffer exists before the capture starts
+    rng = np.random.default_rng(11)
+    n, k = 1024, 14336  # a down-projection-like shape: split over workgroups when launched eagerly
+    n_ff, kf, n_out = 4096, 1024, 512
+    w = q8.tile(to_dev(random_blocks(rng, n, k, 1e-3)), n, k)
+    wg, wu = (q8.tile(to_dev(random_blocks(rng, n_ff, kf, 1e-3)), n_ff, kf) for _ in range(2))
+    wd = q8.tile(to_dev(random_blocks(rng, n_out, n_ff, 1e-3)), n_out, n_ff)
+    x1 = torch.zeros(k, dtype=torch.float32, device="cuda")
+    x8 = torch.zeros((8, k), dtype=torch.float32, device="cuda")
+    xf = torch.zeros(kf, dtype=torch.float32, device="cuda")
+    res = to_dev(rng.standard_normal(n_out).astype(np.float32))
+
+    def launches():
+        return (q8.gemv_f32(w, x1, n, k), q8.mul_mat(w, x8[:3], n, k), q8.mul_mat(w, x8, n, k), q8.ffn(wg, wu, wd, xf, n_ff, kf, n_out, residual=res))
+
+    def new_inputs(seed):
+        x8.copy_(to_dev(oracle.fill_activations(seed, 8 * k).reshape(8, k)))
+        x1.copy_(x8[5])
+        xf.copy_(to_dev(oracle.fill_activations(seed + 1000, kf)))
+
+    new_inputs(1)
+    launches()  # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = launches()
+    for seed in (2, 3, 4, 5):
+        new_inputs(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [to_host(t).copy() for t in captured]
+        want = [to_host(t) for t in launches()]  # eager: the split forms, with fresh epochs, between the replays
+        torch.cuda.synchronize()
+        for i, (g, e) in enumerate(zip(got[:3], want[:3])):
+            assert rel_l2(g, e) < 2e-6, (seed, i)  # same arithmetic, different cut of K
+        assert rel_l2(got[3], want[3]) <= 1e-3, seed  # a quantizer sits between the FFN's stages
+        assert np.isfinite(got[3]).all()
+    # and against the checker once, so that "equal to eager" cannot hide a common mistake
+    aq = oracle.quantize_rows(to_host(x1))[0]
+    assert rel_l2(got[0], oracle.gemv(to_host(q8.untile(w, n, k)), aq, n, k)) <= REL_L2_TOL
