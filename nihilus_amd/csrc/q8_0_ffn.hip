@@ -17,9 +17,10 @@
 //
 // Progress: workgroups are dispatched in index order within each XCD's share of the grid, and producers all precede
 // consumers, so a waiting consumer never keeps a producer from being scheduled; producers wait for nothing.  The wait
-// is bounded all the same (see gemv_chunk).  Hand-off: a producer publishes its block with device-scope stores, waits
-// for the acknowledgements, then stores the launch's epoch into the block's flag; nothing is reset between launches
-// (epochs only move forward).
+// is bounded all the same (see gemv_chunk).  Hand-off: a producer publishes its block as nine 64-bit words, each the
+// launch's epoch beside 32 bits of the block, with device-scope stores; a consumer reads the words of its slice until
+// all carry the epoch.  One trip through memory each way (with a flag beside the data it was two each way, and under
+// the weight stream every trip costs 2-3 us); nothing is reset between launches (epochs only move forward).
 #include "q8_0_gemv_tiled.h"
 
 namespace nh {
@@ -34,9 +35,7 @@ struct ffn_args {
 	const float* residual; // [n_out] or null
 	float* y; // [n_out]
 	float* gate_up; // scratch: g at [0, n_ff), u at [FFN_MAX_HIDDEN, FFN_MAX_HIDDEN + n_ff), kept for inspection
-	uint32_t* act_q; // scratch: the activation's quants, 8 dwords per block
-	float* act_d; // scratch: its scales
-	unsigned* flags; // scratch: one word per block
+	uint64_t* act_words; // scratch: the activation, PUBLISHED_WORDS {epoch, payload} words per block
 	unsigned epoch;
 	uint64_t* tagged; // scratch: tagged partial sums of the down projection's K split
 	int n_ff, n_out;
@@ -76,11 +75,10 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
 		float acc			   = 0.0f;
 		if constexpr (!LOOP) {
-			acc = gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, nullptr, nullptr, 0, norm);
+			acc = gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, 0, norm);
 		} else {
 			for (int gc = g0; gc < g1; gc += TILES) {
-				acc += gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false, nullptr, nullptr, 0,
-					norm);
+				acc += gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false, 0, norm);
 				__builtin_amdgcn_wave_barrier();
 			}
 		}
@@ -103,15 +101,12 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 			const float4 v = lane < 8 ? *reinterpret_cast<const float4*>(&act_f[4 * lane]) : make_float4(0.f, 0.f, 0.f, 0.f);
 			uint16_t dh;
 			const uint32_t packed = quantize_block_lane(v, &dh);
-			if (lane < 8) {
-				__hip_atomic_store(&a.act_q[strip * 8 + lane], packed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-			}
-			if (lane == 0) {
-				__hip_atomic_store(&a.act_d[strip], half_bits_to_float(dh), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-			}
-			wait_stores_acknowledged();
-			if (lane == 0) {
-				__hip_atomic_store(&a.flags[strip], a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			// lanes 0..7 hold the quants and the block's scale; lane 8 stores the scale: nine self-tagged words, no
+			// acknowledgement to wait for
+			const uint32_t d_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(half_bits_to_float(dh)));
+			if (lane <= 8) {
+				const uint32_t payload = lane < 8 ? packed : d_bits;
+				__hip_atomic_store(&a.act_words[strip * PUBLISHED_WORDS + lane], (static_cast<uint64_t>(a.epoch) << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 			}
 		}
 		return;
@@ -129,12 +124,10 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 	const int row_l		   = gstrip * STRIP_ROWS + (lane & 31);
 	float acc			   = 0.0f;
 	if constexpr (!LOOP) {
-		acc = gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_q, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_c, lane, row_l, a.n_out, false, a.act_d, a.flags,
-			a.epoch);
+		acc = gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_words, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_c, lane, row_l, a.n_out, false, a.epoch);
 	} else {
 		for (int gc = g0; gc < g1; gc += TILES) {
-			acc += gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_q, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_c, lane, row_l, a.n_out, false,
-				a.act_d, a.flags, a.epoch);
+			acc += gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_words, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_c, lane, row_l, a.n_out, false, a.epoch);
 			__builtin_amdgcn_wave_barrier();
 		}
 	}
@@ -230,9 +223,7 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	a.residual	 = residual;
 	a.y			 = y;
 	a.gate_up	 = sc.gate_up;
-	a.act_q		 = sc.act_q;
-	a.act_d		 = sc.act_d;
-	a.flags		 = sc.flags;
+	a.act_words	 = sc.act_words;
 	a.epoch		 = sc.epoch;
 	a.tagged	 = sc.tagged;
 	a.n_ff		 = static_cast<int>(n_ff);

@@ -148,11 +148,11 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	}
 	if constexpr (!LOOP) {
 		// the host picked splits so that g1 - g0 <= TILES: straight-line code, every load of the wave in flight at once
-		acc = gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm, rowpart);
+		acc = gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, 0, norm, rowpart);
 	} else {
 		// K too long for that within the host's scratch limits: walk the range in chunks of TILES groups
 		for (int gc = g0; gc < g1; gc += TILES) {
-			acc += gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, nullptr, nullptr, 0, norm, rowpart);
+			acc += gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, 0, norm, rowpart);
 			__builtin_amdgcn_wave_barrier(); // the next chunk overwrites this wave's LDS slice
 		}
 	}
@@ -207,7 +207,7 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	gemv_scratch& sc = per_device[dev];
 	if (!sc.tagged) {
 		void* p			   = nullptr;
-		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * (8 + 1 + 1) * 4 + (FFN_MAX_HIDDEN / QK) * BLOCK_BYTES;
+		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS * 8 + (FFN_MAX_HIDDEN / QK) * BLOCK_BYTES;
 		e				   = hipMalloc(&p, bytes);
 		if (e != hipSuccess) {
 			return e;
@@ -219,13 +219,11 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 		}
 		sc.tagged  = static_cast<uint64_t*>(p);
 		sc.gate_up = reinterpret_cast<float*>(sc.tagged + static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS);
-		sc.act_q	= reinterpret_cast<uint32_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
-		sc.act_d	= reinterpret_cast<float*>(sc.act_q + (FFN_MAX_HIDDEN / STRIP_ROWS) * 8);
-		sc.flags	= reinterpret_cast<unsigned*>(sc.act_d + FFN_MAX_HIDDEN / STRIP_ROWS);
-		sc.act_blocks = reinterpret_cast<uint8_t*>(sc.flags + FFN_MAX_HIDDEN / STRIP_ROWS); // 16-byte aligned: every part before it is a multiple of 16 bytes
+		sc.act_words  = reinterpret_cast<uint64_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
+		sc.act_blocks = reinterpret_cast<uint8_t*>(sc.act_words + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS); // 16-byte aligned: every part before it is a multiple of 16 bytes
 	}
 	if (next_epoch) {
-		++sc.epoch; // flags start at zero and the first epoch handed out is 1
+		++sc.epoch; // tags start at zero and the first epoch handed out is 1
 		if (sc.epoch == 0) {
 			++sc.epoch;
 		}

@@ -22,13 +22,16 @@ enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
 // XMODE says where the activation slice comes from:
 //   X_BLOCKS    packed Q8_0 blocks (xin), re-aligned into LDS;
 //   X_F32       fp32 values (xin), quantized on the spot;
-//   X_PUBLISHED quantized blocks that OTHER workgroups of the same launch produce (xin = quants, 8 dwords per block;
-//               xin2 = fp32 scales, one per block): the wave first puts all its weight loads in flight, then waits
-//               until the 4 * cnt blocks of its slice carry `epoch` in `flags` (one word per block), then reads them
-//               with device-scope loads.  The wait is bounded: after FLAG_SPIN_LIMIT polls the wave gives up and
-//               returns NaN, so the kernel always drains.
+//   X_PUBLISHED quantized blocks that OTHER workgroups of the same launch produce.  xin = PUBLISHED_WORDS 64-bit words
+//               per block, each {epoch, payload}: eight dwords of quants and the fp32 scale.  A 64-bit store is seen
+//               whole or not at all, so the data carries its own "ready" mark: the producer needs no acknowledgement
+//               and no flag, the consumer no second read.  The wave first puts all its weight loads in flight, then
+//               reads the 4 * cnt blocks of its slice with device-scope loads until every word carries `epoch`.  The
+//               wait is bounded: after PUBLISHED_SPIN_LIMIT polls the wave gives up and returns NaN, so the kernel
+//               always drains.
 enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2 };
-constexpr int FLAG_SPIN_LIMIT = 1 << 20;
+constexpr int PUBLISHED_SPIN_LIMIT = 1 << 20;
+constexpr int PUBLISHED_WORDS	   = 9; // per block: quant dwords 0..7, then the scale
 
 // RMS norm * weight in front of the quantizer (X_F32 only).  The row's scale needs every element.  The fixed order
 // of the sum of squares (rms_run_* in q8_0_device.h) cuts the row into 16 runs exactly as an unsplit launch cuts K over
@@ -78,7 +81,7 @@ __device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, co
 // hand over between workgroups.
 template<int TILES, int XMODE, int DUMP, bool NORM, int CNT, int RS = 1>
 __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int groups,
-	int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2, const unsigned* __restrict__ flags, unsigned epoch, gemv_norm* norm, int rowpart = 0) {
+	int lane, int row, int N, bool dump_this_strip, unsigned epoch, gemv_norm* norm, int rowpart = 0) {
 	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
 	static_assert(RS == 1 || RS == 2 || RS == 4, "a strip splits into 1, 2 or 4 row parts");
@@ -143,44 +146,47 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 		}
 	}
 
-	// ---- 2b. the slice comes from this launch's own producers: wait for them, then fetch it ----
+	// ---- 2b. the slice comes from this launch's own producers: read it until every word is this launch's ----
 	bool timed_out = false;
 	if constexpr (XMODE == X_PUBLISHED) {
-		const unsigned* f = flags + gc * GROUP_BLOCKS;
-		const int n_flags = cnt * GROUP_BLOCKS;
-		int spins		  = 0;
+		// device-scope loads: the producers ran on other XCDs, whose L2 this one does not snoop
+		const uint64_t* pw	   = static_cast<const uint64_t*>(xin) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * PUBLISHED_WORDS);
+		constexpr int PW_LOADS = (TILES * GROUP_BLOCKS * PUBLISHED_WORDS + 63) / 64;
+		const int n_words	   = cnt * GROUP_BLOCKS * PUBLISHED_WORDS;
+		uint64_t pv[PW_LOADS];
+		int spins = 0;
 		for (;;) {
-			const unsigned seen = lane < n_flags ? __hip_atomic_load(f + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : epoch;
-			if (__builtin_amdgcn_ballot_w64(seen != epoch) == 0) {
+			bool fresh = true;
+#pragma unroll
+			for (int i = 0; i < PW_LOADS; ++i) {
+				const int v = lane + 64 * i;
+				pv[i]		= v < n_words ? __hip_atomic_load(pw + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : (static_cast<uint64_t>(epoch) << 32);
+			}
+#pragma unroll
+			for (int i = 0; i < PW_LOADS; ++i) {
+				fresh = fresh && static_cast<unsigned>(pv[i] >> 32) == epoch;
+			}
+			if (__builtin_amdgcn_ballot_w64(!fresh) == 0) {
 				break;
 			}
-			if (++spins >= FLAG_SPIN_LIMIT) {
+			if (++spins >= PUBLISHED_SPIN_LIMIT) {
 				timed_out = true;
 				break;
 			}
-			__builtin_amdgcn_s_sleep(16);
+			__builtin_amdgcn_s_sleep(8);
 		}
-		asm volatile("" ::: "memory"); // the data loads below stay behind the flag loads above
-		// device-scope loads: the producers ran on other XCDs, whose L2 this one does not snoop
-		const uint32_t* pq = static_cast<const uint32_t*>(xin) + gc * (GROUP_BLOCKS * 8);
-		const float* pd	   = static_cast<const float*>(xin2) + gc * GROUP_BLOCKS;
-		constexpr int PQ_LOADS = (TILES * 32 + 63) / 64; // 32 dwords per group
-		uint32_t qv[PQ_LOADS];
 #pragma unroll
-		for (int i = 0; i < PQ_LOADS; ++i) {
+		for (int i = 0; i < PW_LOADS; ++i) {
 			const int v = lane + 64 * i;
-			qv[i]		= v < cnt * 32 ? __hip_atomic_load(pq + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-		}
-		const float dv = lane < n_flags ? __hip_atomic_load(pd + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
-#pragma unroll
-		for (int i = 0; i < PQ_LOADS; ++i) {
-			const int v = lane + 64 * i;
-			if (v < cnt * 32) {
-				*reinterpret_cast<uint32_t*>(xs_q + 4 * v) = qv[i]; // block v/8 at 32*(v/8), dword v%8
+			if (v < n_words) {
+				const int blk = v / PUBLISHED_WORDS, j = v - blk * PUBLISHED_WORDS;
+				const uint32_t payload = static_cast<uint32_t>(pv[i]);
+				if (j < 8) {
+					*reinterpret_cast<uint32_t*>(xs_q + blk * QK + 4 * j) = payload;
+				} else {
+					xs_d[blk] = __uint_as_float(payload);
+				}
 			}
-		}
-		if (lane < n_flags) {
-			xs_d[lane] = dv;
 		}
 	}
 
@@ -303,12 +309,11 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 
 template<int TILES, int XMODE, int DUMP, bool NORM = false, int RS = 1>
 __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
-	int groups, int lane, int row, int N, bool dump_this_strip, const void* __restrict__ xin2 = nullptr, const unsigned* __restrict__ flags = nullptr, unsigned epoch = 0,
-	gemv_norm* norm = nullptr, int rowpart = 0) {
+	int groups, int lane, int row, int N, bool dump_this_strip, unsigned epoch = 0, gemv_norm* norm = nullptr, int rowpart = 0) {
 #define NH_CHUNK_CASE(C)                                                                                                                                              \
 	case C:                                                                                                                                                           \
 		if constexpr (C <= TILES) {                                                                                                                                   \
-			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0), RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm, rowpart); \
+			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0), RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart); \
 		}                                                                                                                                                             \
 		break;
 	switch (cnt) { // wave-uniform
@@ -320,7 +325,7 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 			break;
 	}
 #undef NH_CHUNK_CASE
-	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0, RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, xin2, flags, epoch, norm, rowpart); // an idle wave (still takes part in barriers)
+	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0, RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart); // an idle wave (still takes part in barriers)
 }
 
 // K split over several workgroups: each publishes the 32 partial sums of its share, tagged with the launch's epoch
@@ -376,9 +381,7 @@ constexpr int FFN_MAX_HIDDEN		= 65536; // rows of the gate / up projections in a
 struct gemv_scratch {
 	uint64_t* tagged   = nullptr; // [GEMV_MAX_SPLIT_UNITS][32] {epoch, partial sum}
 	float* gate_up	   = nullptr; // [2][FFN_MAX_HIDDEN]: the gate and up outputs (kept for inspection only)
-	uint32_t* act_q	   = nullptr; // [FFN_MAX_HIDDEN / 32][8]: the quantized activation of the down projection, 8 dwords per block
-	float* act_d	   = nullptr; // [FFN_MAX_HIDDEN / 32]: its scales (the fp16-rounded value, widened)
-	unsigned* flags	   = nullptr; // [FFN_MAX_HIDDEN / 32]: the epoch of the launch that last published the block
+	uint64_t* act_words = nullptr; // [FFN_MAX_HIDDEN / 32][PUBLISHED_WORDS] {epoch, payload}: the quantized activation of the down projection
 	uint8_t* act_blocks = nullptr; // [FFN_MAX_HIDDEN / 32] packed 34-byte blocks: the activation of the three-launch form used under graph capture
 	unsigned epoch	   = 0; // with next_epoch = true: a value no earlier launch on this device has used
 };
