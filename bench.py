@@ -4,13 +4,16 @@
 Workload (the configuration the metric is quoted on): the LLaMA-3-8B FFN decode mat-vecs at batch 1 --
 gate and up, Q8_0 W [14336 x 4096], and down, Q8_0 W [4096 x 14336] -- with the activation quantize inside
 the step.  One step = quantize(x[4096]) -> gate, up ; quantize(h[14336]) -> down, enqueued by one native
-batch call, which runs it as two launches of the streaming mat-vec kernel (gate+up share x and go out as one
-launch; the quantize happens inside the kernel).  Steps rotate over `--layers` distinct weight sets (default 16 x 187 MB = 3 GB) so that every
+batch call.  The three mat-vecs of this configuration are independent (each has its own seeded input), which the
+batch runner sees from their input and output ranges, so it runs them as ONE launch of the grouped mat-vec kernel
+(every matrix cut as its own launch would cut it, the quantize inside the kernel).  The default run also reports the
+same step as two launches (gate+up, then down: what a caller gets who marks the down projection as ordered after
+the others) and as the one-launch FFN with the real dependency inside (down fed by SiLU(gate) * up).  Steps rotate over `--layers` distinct weight sets (default 16 x 187 MB = 3 GB) so that every
 byte comes from HBM and not from the 256 MB last-level cache.  Inputs are resident in HBM before the timed
 region; synthetic data from the library's counter-based generator (seed 0).
 
 Prints ONE JSON line.  `value` = algorithmic bytes per step / wall time per step.  `roofline` is for the
-dominant kernel (the tiled mat-vec): algorithmic bytes per launch / its average duration, measured live with
+dominant kernel (the grouped mat-vec): algorithmic bytes per launch / its average duration, measured live with
 start/stop timestamps carried in each launch's own dispatch packet.  `cpu_baseline` is the AVX2 restatement
 of the reference arithmetic on the host's cores (a reported number, not the target).
 """
@@ -28,11 +31,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 GATE_N, HIDDEN, FFN = 14336, 4096, 14336
-# HBM bytes per launch of the dominant kernel, mean over the step's two launches: FETCH_SIZE and WRITE_SIZE from two
+# HBM bytes per launch of the dominant kernel (mean over the step's launches): FETCH_SIZE and WRITE_SIZE from two
 # rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for a plain 64 MiB copy
 # (FETCH_SIZE x 1.99927, WRITE_SIZE x 1.0).  A hardware-counter figure cannot be taken live; this is the recorded one.
 # Keyed by --ffn-mode; None = not measured yet for that mode.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"batch": 93887437, "fused": 187808256}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"group": None, "two": 93887437, "fused": 187808256}
 
 
 def weight_bytes(n: int, k: int) -> int:
@@ -64,10 +67,11 @@ def main() -> int:
     ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover", "llama70b"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
-    ap.add_argument("--ffn-mode", choices=["batch", "fused"], default="batch",
-                    help="batch (default): the step's three mat-vecs through nh_q8_0_mul_mat_batch as two launches, the down projection fed from a "
-                    "resident fp32 vector (mat-vecs only, as the metric is defined).  fused: the step as one launch (nh_q8_0_ffn_f32: gate, up, "
-                    "SiLU*up, down), which the default run reports beside the headline as `ffn_one_launch`")
+    ap.add_argument("--ffn-mode", choices=["group", "two", "fused"], default="group",
+                    help="group (default): the step's three mat-vecs through nh_q8_0_mul_mat_batch, the down projection fed from a resident fp32 "
+                    "vector (mat-vecs only, as the metric is defined); the runner finds them independent and issues one grouped launch.  two: the same "
+                    "with the down projection marked ordered: gate+up, then down, two launches.  fused: the step as one launch with the real "
+                    "dependency inside (nh_q8_0_ffn_f32: gate, up, SiLU*up, down).  The default run reports the other two beside the headline")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode-step leg (8 GB of weights)")
     ap.add_argument("--decode-tokens", type=int, default=200, help="timed tokens of the decode-step leg")
     ap.add_argument("--roofline-steps", type=int, default=0, help="steps of the per-kernel timing pass (default: min(steps, 1000))")
@@ -131,10 +135,16 @@ def main() -> int:
         ops[2] = _lib.MulMatOp(mats[2].data_ptr(), h.data_ptr(), y_down.data_ptr(), 1, HIDDEN, FFN, 0, 0)
         op_lists.append(ops)
 
+    def set_ordered(flag: int) -> None:
+        for ops in op_lists:
+            ops[2].ordered = flag
+
     batch = lib.nh_q8_0_mul_mat_batch
     ws_ptr, ws_n = ws.data_ptr(), ws.numel()
 
-    fused = args.ffn_mode == "fused"
+    mode = args.ffn_mode
+    fused = mode == "fused"
+    set_ordered(1 if mode == "two" else 0)
     ffn = lib.nh_q8_0_ffn_f32
     ptrs = [(m[0].data_ptr(), m[1].data_ptr(), m[2].data_ptr()) for m in layers]
     x_ptr, y_ptr = x.data_ptr(), y_down.data_ptr()
@@ -150,12 +160,16 @@ def main() -> int:
                 _lib.check("nh_q8_0_ffn_f32" if fused else "nh_q8_0_mul_mat_batch", rc)
 
     # algorithmic bytes of the step: every weight block once, the fp32 activation rows read, the fp32 outputs written.
-    # batch mode: two launches, gate+up (shared x) and down, each with its quantize inside.  fused mode: one launch; the
-    # gate/up outputs (2 x 57 KB) stay inside the launch and are not counted.
-    if fused:
-        launch_bytes_list = [fused_launch_bytes([GATE_N, GATE_N], HIDDEN) - 8 * GATE_N + fused_launch_bytes([HIDDEN], FFN) - 4 * FFN]
-    else:
-        launch_bytes_list = [fused_launch_bytes([GATE_N, GATE_N], HIDDEN), fused_launch_bytes([HIDDEN], FFN)]
+    # group: one launch of all three; two: gate+up (shared x), then down; each with its quantize inside.  fused: one launch;
+    # the gate/up outputs (2 x 57 KB) stay inside the launch and are not counted.
+    def launch_bytes_of(m: str) -> list[int]:
+        if m == "fused":
+            return [fused_launch_bytes([GATE_N, GATE_N], HIDDEN) - 8 * GATE_N + fused_launch_bytes([HIDDEN], FFN) - 4 * FFN]
+        if m == "two":
+            return [fused_launch_bytes([GATE_N, GATE_N], HIDDEN), fused_launch_bytes([HIDDEN], FFN)]
+        return [fused_launch_bytes([GATE_N, GATE_N], HIDDEN) + fused_launch_bytes([HIDDEN], FFN)]
+
+    launch_bytes_list = launch_bytes_of(mode)
     step_bytes = sum(launch_bytes_list)
 
     # ---------------------------------------------------------------- warm-up, then EXACTLY --steps timed steps
@@ -197,7 +211,8 @@ def main() -> int:
         "data": "synthetic",
         "config": {
             "workload": "LLaMA-3-8B FFN decode GEMVs, batch 1: gate+up Q8_0 [14336x4096], down Q8_0 [4096x14336], activation quantize included"
-            + (", SiLU(gate)*up feeding down, one launch per step" if fused else ", two launches per step"),
+            + {"fused": ", SiLU(gate)*up feeding down, one launch per step", "two": ", two launches per step (gate+up, down)",
+               "group": ", three independent mat-vecs grouped into one launch per step"}[mode],
             "weight_sets_rotated": L,
             "bytes_per_step": step_bytes,
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
@@ -205,14 +220,16 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": ("nh::ffn_decode_kernel<TILES=2> (gate, up and down mat-vecs of the step as one 187 MB launch, activation quantize and SiLU*up inside)"
-                       if fused else "nh::gemv_tiled_kernel<TILES, XF32=true> (streaming mat-vec with the activation quantize inside; "
-                       "two launches per step: gate+up as one 125 MB launch, down as one 62 MB launch)"),
+            "kernel": {"fused": "nh::ffn_decode_kernel<TILES=4> (gate, up and down mat-vecs of the step as one 187 MB launch, activation quantize and SiLU*up inside)",
+                       "two": "nh::gemv_tiled_kernel<TILES=2, XF32=true> (streaming mat-vec with the activation quantize inside; "
+                              "two launches per step: gate+up as one 125 MB launch, down as one 62 MB launch)",
+                       "group": "nh::gemv_group_kernel<TILES=2> (streaming mat-vec over independent matrices with the activation quantize inside; "
+                                "gate, up and down as one 187 MB launch)"}[mode],
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH[args.ffn_mode],
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH[mode],
             "bytes_per_launch": launch_bytes,
             "avg_launch_us": round(avg_ms * 1e3, 3),
             "min_launch_us": round(mn.value * 1e3, 3),
@@ -221,20 +238,28 @@ def main() -> int:
         },
     }
 
-    if not fused:
-        # the same step as ONE launch with the real dependency inside (down fed by silu(gate) * up): reported beside the headline
-        fb = fused_launch_bytes([GATE_N, GATE_N], HIDDEN) - 8 * GATE_N + fused_launch_bytes([HIDDEN], FFN) - 4 * FFN
-        fused = True
-        run_steps(args.warmup)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        run_steps(args.steps, start=args.warmup)
-        torch.cuda.synchronize()
-        f_sec = (time.perf_counter() - t0) / args.steps
-        result["ffn_one_launch"] = {"entry": "nh_q8_0_ffn_f32", "ms_per_step": round(f_sec * 1e3, 6), "GBs": round(fb / f_sec / 1e9, 1),
-                                    "pct_of_hbm_peak": round(100.0 * fb / f_sec / 1e9 / HBM_PEAK_GBS, 2), "bytes_per_step": fb,
-                                    "outputs_finite": bool(torch.isfinite(y_down).all())}
-        fused = False
+    if mode == "group":
+        # the same step the other two ways, timed the same way, beside the headline
+        def timed_other(m: str) -> tuple[float, bool]:
+            nonlocal fused
+            fused = m == "fused"
+            set_ordered(1 if m == "two" else 0)
+            run_steps(args.warmup)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            run_steps(args.steps, start=args.warmup)
+            torch.cuda.synchronize()
+            sec = (time.perf_counter() - t) / args.steps
+            ok = bool(torch.isfinite(y_down).all())
+            fused = False
+            set_ordered(0)
+            return sec, ok
+
+        for m, key, entry in (("two", "ffn_two_launches", "nh_q8_0_mul_mat_batch, down marked ordered"), ("fused", "ffn_one_launch", "nh_q8_0_ffn_f32")):
+            sec, ok = timed_other(m)
+            nb = sum(launch_bytes_of(m))
+            result[key] = {"entry": entry, "ms_per_step": round(sec * 1e3, 6), "GBs": round(nb / sec / 1e9, 1), "pct_of_hbm_peak": round(100.0 * nb / sec / 1e9 / HBM_PEAK_GBS, 2),
+                           "bytes_per_step": nb, "outputs_finite": ok}
 
     del layers, op_lists
     torch.cuda.empty_cache()
@@ -417,9 +442,13 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
 def decode_step(tokens: int) -> dict:
     """The second half of the metric: one decode step of a LLaMA-3-8B-shaped model with every mat-mul in Q8_0
     (32 layers x {q, k, v, o, gate, up, down} + lm_head, random weights from the generator, fp32 N(0,1) inputs
-    per projection; mat-muls only, no attention/norm math).  One token = one native batch call of 225 projections,
-    which the runner issues as 129 launches (q/k/v and gate/up fused).  All 8 GB of weights are distinct, so every
-    token streams them from HBM."""
+    per projection; mat-muls only, no attention/norm math).  One token = one native batch call of 225 projections.
+    Headline figures: the entries that a model's data flow orders after their predecessors (q after the previous
+    layer, o after the attention, gate after o, down after gate/up, lm_head after the last layer) carry the `ordered`
+    mark, so the runner issues 129 launches (q/k/v and gate/up share one each).  `independent` is the same list without
+    the marks: the inputs of this configuration are resident vectors, the runner sees from the pointers that a layer's
+    seven projections do not depend on each other, and issues one grouped launch per layer.  All 8 GB of weights are
+    distinct, so every token streams them from HBM."""
     import torch
 
     from nihilus_amd import _lib, q8_0
@@ -448,6 +477,7 @@ def decode_step(tokens: int) -> dict:
     outs = {name: torch.empty(n, dtype=torch.float32, device=dev) for name, n, _ in shapes}
     logits = torch.empty(V, dtype=torch.float32, device=dev)
     weights = []
+    model_order = []  # per entry: starts after its predecessors in a model's data flow
     ops = (_lib.MulMatOp * (LAYERS * 7 + 1))()
     i = 0
     wbytes = 0
@@ -457,10 +487,12 @@ def decode_step(tokens: int) -> dict:
             weights.append(w)
             wbytes += n * (k // 32) * 34
             ops[i] = _lib.MulMatOp(w.data_ptr(), xin[name].data_ptr(), outs[name].data_ptr(), 1, n, k, 1 if name in ("k", "v", "up") else 0, 0)
+            model_order.append(1 if name in ("q", "o", "gate", "down") else 0)
             i += 1
     w_head = make(V, H)
     wbytes += V * (H // 32) * 34
     ops[i] = _lib.MulMatOp(w_head.data_ptr(), x_head.data_ptr(), logits.data_ptr(), 1, V, H, 0, 0)
+    model_order.append(1)
     n_ops = i + 1
     ws = torch.empty(256, dtype=torch.uint8, device=dev)
 
@@ -469,14 +501,24 @@ def decode_step(tokens: int) -> dict:
         if rc != 0:
             _lib.check("nh_q8_0_mul_mat_batch", rc)
 
-    for _ in range(10):
+    def timed(marks: bool) -> tuple[float, int]:
+        for j in range(n_ops):
+            ops[j].ordered = model_order[j] if marks else 0
+        for _ in range(10):
+            token()
+        torch.cuda.synchronize()
+        _lib.check("nh_profile_begin", lib.nh_profile_begin(1, 512))
         token()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(tokens):
-        token()
-    torch.cuda.synchronize()
-    sec = (time.perf_counter() - t0) / tokens
+        tot, cnt, mn, mx = C.c_double(), C.c_int64(), C.c_double(), C.c_double()
+        _lib.check("nh_profile_end", lib.nh_profile_end(C.byref(tot), C.byref(cnt), C.byref(mn), C.byref(mx)))
+        t0 = time.perf_counter()
+        for _ in range(tokens):
+            token()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / tokens, cnt.value
+
+    sec, launches = timed(True)
+    sec_i, launches_i = timed(False)
     return {
         "tok_s": round(1.0 / sec, 1),
         "ms_per_token": round(sec * 1e3, 4),
@@ -484,9 +526,12 @@ def decode_step(tokens: int) -> dict:
         "weight_GBs": round(wbytes / sec / 1e9, 1),
         "pct_of_hbm_peak": round(100.0 * wbytes / sec / 1e9 / HBM_PEAK_GBS, 2),
         "projections_per_token": n_ops,
-        "launches_per_token": LAYERS * 4 + 1,
+        "launches_per_token": launches,
         "tokens_timed": tokens,
         "outputs_finite": bool(torch.isfinite(logits).all()),
+        "independent": {"tok_s": round(1.0 / sec_i, 1), "ms_per_token": round(sec_i * 1e3, 4), "pct_of_hbm_peak": round(100.0 * wbytes / sec_i / 1e9 / HBM_PEAK_GBS, 2),
+                        "launches_per_token": launches_i,
+                        "note": "same list without the ordered marks: a layer's seven projections read resident vectors here, so they go out as one grouped launch"},
     }
 
 

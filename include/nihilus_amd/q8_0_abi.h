@@ -167,6 +167,17 @@ int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* co
 int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* norm_weight, float eps, const float* residual, float* y,
 	int64_t N_ff, int64_t K, int64_t N_out, void* stream);
 
+/* `count` INDEPENDENT mat-vecs, each with its own fp32 activation row, K and N (host arrays of device pointers and sizes;
+ * host_residual or any entry of it may be NULL): y_i = W_i . quantize(x_i) [+ residual_i].  None of them may read or
+ * overwrite what another one writes (a residual that is the op's own y is fine); given that, they run as one launch per up to
+ * eight matrices instead of one each, so the ~3 us a launch spends filling and draining the chip are paid once per group.
+ * Each matrix is cut as its own launch would cut it, so results equal those of separate nh_q8_0_gemv_tiled_f32 calls (bit for
+ * bit unless the separate call would split a small matrix by rows, then to fp32 summation order).  No counterpart in the
+ * reference, whose per-op dispatch (cpu/avx_2.hpp:1296-1444) runs one mul_mat per call; nh_q8_0_mul_mat_batch uses it for
+ * neighbouring entries it can prove independent. */
+int nh_q8_0_gemv_tiled_group_f32(const void* const* host_W_tiled, const float* const* host_x, float* const* host_y, const float* const* host_residual, const int64_t* host_N,
+	const int64_t* host_K, int64_t count, void* stream);
+
 /* Mat-mat (prefill, prompt_eval_time) ----------------------------------------------------------- */
 
 /* C[m*N + n] (n fastest, ggml's dst[ir1*nr0 + ir0], cpu/avx_2.hpp:4934) = the same dot for activation
@@ -195,19 +206,25 @@ int nh_q8_0_mul_mat_residual(const void* W_tiled, const float* x, const float* r
 
 /* One entry of a batch: y[M][N] = mul_mat(W_tiled [N x K], x fp32 [M][K]).  reuse_quantized_x != 0 lets the runner
  * skip the quantize when the previous entry quantized the same x pointer with the same M and K (q/k/v share the
- * normed hidden state, gate/up share the FFN input: infra/core_traits.hpp:575-594, :976-986). */
+ * normed hidden state, gate/up share the FFN input: infra/core_traits.hpp:575-594, :976-986).
+ * ordered != 0: the entry starts only after every earlier entry has finished, whatever its pointers say (set it when
+ * the entry depends on earlier ones through memory other than their x and y ranges).  With ordered == 0 the runner may
+ * put neighbouring M == 1 entries into one launch when it can see from their x and y ranges that none reads or
+ * overwrites what another writes; entries whose ranges do overlap always run in list order. */
 typedef struct nh_q8_0_mul_mat_op {
 	const void* W_tiled;
 	const float* x;
 	float* y;
 	int64_t M, N, K;
 	int32_t reuse_quantized_x;
-	int32_t reserved;
+	int32_t ordered;
 } nh_q8_0_mul_mat_op;
 /* Enqueues `count` mul_mat operations in order on one stream from native code: one call per decode step instead
  * of one per projection (the per-block fold of cuda/thread_pool.hpp:46-67 over the three mega cores).  host_ops is
  * host memory, read before return.  workspace must hold the largest nh_q8_0_mul_mat_workspace_bytes(M, K) of the
- * list; entries run in stream order, so sharing it is safe.  All entries are validated before the first launch. */
+ * list; entries that use it run in stream order, so sharing it is safe.  The result is that of running the entries one
+ * after another in list order (independent neighbours may share a launch, see nh_q8_0_mul_mat_op).  All entries are
+ * validated before the first launch. */
 int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Per-kernel timing (instrumentation) ----------------------------------------------------------- */

@@ -5,6 +5,7 @@
 #include "q8_0_device.h"
 
 #include <cstring>
+#include <vector>
 
 namespace {
 
@@ -382,6 +383,36 @@ int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* co
 	int64_t K, void* stream) {
 	NH_REQUIRE(norm_weight || K == 0 || count == 0, NH_ERR_NULL_POINTER);
 	return gemv_multi_common(host_W_tiled, host_y, host_N, count, x, norm_weight, eps, K, stream);
+}
+
+int nh_q8_0_gemv_tiled_group_f32(const void* const* host_W_tiled, const float* const* host_x, float* const* host_y, const float* const* host_residual, const int64_t* host_N,
+	const int64_t* host_K, int64_t count, void* stream) {
+	NH_REQUIRE(count >= 0 && count <= 4096, NH_ERR_ARGUMENT);
+	if (count == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(host_W_tiled && host_x && host_y && host_N && host_K, NH_ERR_NULL_POINTER);
+	std::vector<nh::gemv_group_op> ops;
+	ops.reserve(static_cast<size_t>(count));
+	for (int64_t i = 0; i < count; ++i) {
+		NH_TRY(check_shape(host_N[i], 0, host_K[i], true));
+		if (host_N[i] == 0) {
+			continue;
+		}
+		const float* res = host_residual ? host_residual[i] : nullptr;
+		NH_REQUIRE(host_y[i], NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(host_y[i]) && aligned16(res), NH_ERR_ALIGNMENT);
+		if (host_K[i] > 0) {
+			NH_REQUIRE(host_W_tiled[i] && host_x[i], NH_ERR_NULL_POINTER);
+			NH_REQUIRE(aligned16(host_W_tiled[i]) && aligned16(host_x[i]), NH_ERR_ALIGNMENT);
+		}
+		ops.push_back({ host_W_tiled[i], host_x[i], host_y[i], res, host_N[i], host_K[i] });
+	}
+	if (ops.empty()) {
+		return NH_OK;
+	}
+	NH_TRY(require_device());
+	return from_hip(nh::launch_gemv_independent(ops.data(), static_cast<int64_t>(ops.size()), as_stream(stream)));
 }
 
 int nh_q8_0_prepare(void) {

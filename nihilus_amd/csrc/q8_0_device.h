@@ -253,6 +253,20 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	int64_t K, int64_t n_out, hipStream_t s);
 hipError_t copy_ffn_gate_up(float* gate_out, float* up_out, int64_t n_ff, hipStream_t s);
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w = nullptr, float norm_eps = 0.0f);
+// Mat-vecs that share nothing (own activation row, K, N) as one launch, up to GEMV_GROUP_MAX of them; the caller vouches that
+// none of them reads or overwrites another's output.  launch_gemv_group takes matrices whose waves own at most four groups
+// (anything plan_gemv can cut that way); launch_gemv_independent takes any list and falls back to single launches for the rest.
+constexpr int GEMV_GROUP_MAX = 8;
+struct gemv_group_op {
+	const void* W; // tiled
+	const float* x; // fp32 [K]
+	float* y; // fp32 [N]
+	const float* residual; // fp32 [N] or null
+	int64_t N, K;
+};
+hipError_t launch_gemv_group(const gemv_group_op* ops, int count, hipStream_t s);
+hipError_t launch_gemv_independent(const gemv_group_op* ops, int64_t count, hipStream_t s);
+
 // 2 <= M <= GEMV_ROWS_MAX fp32 activation rows against one tiled weight matrix: the streaming mat-vec with M dot products per
 // weight tile, quantize included (q8_0_gemv_rows.hip).  y is [M][N].
 constexpr int64_t GEMV_ROWS_MAX = 3;

@@ -149,24 +149,62 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 			continue;
 		}
 		if (op.M == 1) {
-			// decode: the quantize lives inside the mat-vec kernel; neighbours that share x and K become one launch
-			const void* w[nh::GEMV_MAX_SEGMENTS];
-			float* y[nh::GEMV_MAX_SEGMENTS];
-			int64_t n[nh::GEMV_MAX_SEGMENTS];
-			int64_t g = 0;
-			while (i + g < count && g < nh::GEMV_MAX_SEGMENTS) {
+			// decode: the quantize lives inside the mat-vec kernel.  The longest run of M == 1 entries of which none reads or
+			// overwrites what an earlier one of the run writes (seen from their x and y ranges) and none asks to be ordered
+			// goes out together: the result is that of running them in list order, whatever runs side by side.
+			auto overlap = [](const float* a, int64_t na, const float* b, int64_t nb) {
+				const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+				return a0 < b0 + static_cast<uintptr_t>(nb) * 4 && b0 < a0 + static_cast<uintptr_t>(na) * 4;
+			};
+			int64_t g	= 1;
+			bool shared = true; // every entry of the run has the first one's x and K
+			while (i + g < count) {
 				const nh_q8_0_mul_mat_op& o = host_ops[i + g];
-				if (o.M != 1 || o.N == 0 || o.x != op.x || o.K != op.K || (g > 0 && !o.reuse_quantized_x)) {
+				if (g >= 64 || o.M != 1 || o.N == 0 || o.ordered) { // 64: the hazard check is quadratic in the run length
 					break;
 				}
-				w[g] = o.W_tiled;
-				y[g] = o.y;
-				n[g] = o.N;
+				bool hazard = false;
+				for (int64_t e = 0; e < g && !hazard; ++e) {
+					const nh_q8_0_mul_mat_op& p = host_ops[i + e];
+					hazard = overlap(o.y, o.N, p.y, p.N) || overlap(o.y, o.N, p.x, p.K) || overlap(o.x, o.K, p.y, p.N);
+				}
+				if (hazard) {
+					break;
+				}
+				shared = shared && o.x == op.x && o.K == op.K;
 				++g;
 			}
-			const int rc = nh_q8_0_gemv_tiled_multi_f32(w, y, n, g, op.x, op.K, stream);
-			if (rc != NH_OK) {
-				return rc;
+			if (shared && g <= nh::GEMV_MAX_SEGMENTS) {
+				// neighbours that share x and K (q/k/v, gate/up) and nothing else to go with them: segments of one mat-vec launch
+				const void* w[nh::GEMV_MAX_SEGMENTS];
+				float* y[nh::GEMV_MAX_SEGMENTS];
+				int64_t n[nh::GEMV_MAX_SEGMENTS];
+				for (int64_t e = 0; e < g; ++e) {
+					w[e] = host_ops[i + e].W_tiled;
+					y[e] = host_ops[i + e].y;
+					n[e] = host_ops[i + e].N;
+				}
+				const int rc = nh_q8_0_gemv_tiled_multi_f32(w, y, n, g, op.x, op.K, stream);
+				if (rc != NH_OK) {
+					return rc;
+				}
+			} else {
+				std::vector<const void*> w(static_cast<size_t>(g));
+				std::vector<const float*> x(static_cast<size_t>(g));
+				std::vector<float*> y(static_cast<size_t>(g));
+				std::vector<int64_t> n(static_cast<size_t>(g)), k(static_cast<size_t>(g));
+				for (int64_t e = 0; e < g; ++e) {
+					const nh_q8_0_mul_mat_op& o = host_ops[i + e];
+					w[static_cast<size_t>(e)]	= o.W_tiled;
+					x[static_cast<size_t>(e)]	= o.x;
+					y[static_cast<size_t>(e)]	= o.y;
+					n[static_cast<size_t>(e)]	= o.N;
+					k[static_cast<size_t>(e)]	= o.K;
+				}
+				const int rc = nh_q8_0_gemv_tiled_group_f32(w.data(), x.data(), y.data(), nullptr, n.data(), k.data(), g, stream);
+				if (rc != NH_OK) {
+					return rc;
+				}
 			}
 			i += g;
 			continue;

@@ -170,6 +170,34 @@ def gemv_f32(w_tiled: list[torch.Tensor] | torch.Tensor, x: torch.Tensor, n: lis
     return ys[0] if single else ys
 
 
+def gemv_group_f32(w_tiled: list[torch.Tensor], xs: list[torch.Tensor], ns: list[int], ks: list[int], residuals: list[torch.Tensor | None] | None = None,
+                   outs: list[torch.Tensor] | None = None) -> list[torch.Tensor]:
+    """Independent mat-vecs, each with its own activation row, k and n, in as few launches as their shapes allow (one per up
+    to eight matrices).  The caller vouches that no output is another op's input, residual or output."""
+    import ctypes as C
+
+    cnt = len(w_tiled)
+    if not (len(xs) == len(ns) == len(ks) == cnt) or (residuals is not None and len(residuals) != cnt) or (outs is not None and len(outs) != cnt):
+        raise ValueError("one x, n and k (and residual, out) per weight")
+    xs = [_dev(x, torch.float32, "x") for x in xs]
+    for w, x, n, k in zip(w_tiled, xs, ns, ks):
+        if x.numel() != k or _dev(w, torch.uint8, "w_tiled").numel() != tiled_bytes(n, k):
+            raise ValueError("operand sizes do not match n x k")
+    ys = [torch.empty(n, dtype=torch.float32, device=xs[0].device) for n in ns] if outs is None else [_dev(o, torch.float32, "out") for o in outs]
+    if any(y.numel() != n for y, n in zip(ys, ns)):
+        raise ValueError("every out must hold n floats")
+    rs = [None] * cnt if residuals is None else [None if r is None else _dev(r, torch.float32, "residual") for r in residuals]
+    if any(r is not None and r.numel() != n for r, n in zip(rs, ns)):
+        raise ValueError("every residual must hold n floats")
+    wp = (C.c_void_p * cnt)(*[w.data_ptr() for w in w_tiled])
+    xp = (C.c_void_p * cnt)(*[x.data_ptr() for x in xs])
+    yp = (C.c_void_p * cnt)(*[y.data_ptr() for y in ys])
+    rp = (C.c_void_p * cnt)(*[None if r is None else r.data_ptr() for r in rs])
+    _lib.check("nh_q8_0_gemv_tiled_group_f32",
+               _lib.lib().nh_q8_0_gemv_tiled_group_f32(wp, xp, yp, rp, (C.c_int64 * cnt)(*ns), (C.c_int64 * cnt)(*ks), cnt, _stream()))
+    return ys
+
+
 def gemv_residual_f32(w_tiled: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, n: int, k: int, out: torch.Tensor | None = None) -> torch.Tensor:
     """y = W . Q(x) + residual in one launch (out may be the residual tensor itself: in-place accumulate)."""
     w_tiled, x, residual = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(x, torch.float32, "x"), _dev(residual, torch.float32, "residual")
