@@ -60,3 +60,47 @@ def test_captured_launches_replay_with_new_inputs(q8, oracle):
     # and against the checker once, so that "equal to eager" cannot hide a common mistake
     aq = oracle.quantize_rows(to_host(x1))[0]
     assert rel_l2(got[0], oracle.gemv(to_host(q8.untile(w, n, k)), aq, n, k)) <= REL_L2_TOL
+
+
+def test_captured_batch_of_independent_mat_vecs(q8, oracle):
+    # a batch call whose entries the runner may group: under capture the short-K ones still share a launch (no per-launch
+    # state when K is not split), the long-K one falls back to its own unsplit launch; replays must follow new inputs
+    import torch
+
+    from nihilus_amd import _lib
+
+    lib = _lib.lib()
+    _lib.check("nh_q8_0_prepare", lib.nh_q8_0_prepare())
+    shapes = [(2048, 1024), (1024, 1024), (512, 14336)]
+    ws = [q8.tile(q8.fill_weight_blocks(90 + i, n, k), n, k) for i, (n, k) in enumerate(shapes)]
+    xs = [torch.zeros(k, dtype=torch.float32, device="cuda") for _, k in shapes]
+    ys = [torch.zeros(n, dtype=torch.float32, device="cuda") for n, _ in shapes]
+    ops = (_lib.MulMatOp * 3)()
+    for i, (n, k) in enumerate(shapes):
+        ops[i] = _lib.MulMatOp(ws[i].data_ptr(), xs[i].data_ptr(), ys[i].data_ptr(), 1, n, k, 0, 0)
+    dummy = torch.empty(256, dtype=torch.uint8, device="cuda")
+
+    def call():
+        _lib.check("nh_q8_0_mul_mat_batch", lib.nh_q8_0_mul_mat_batch(ops, 3, dummy.data_ptr(), dummy.numel(), torch.cuda.current_stream().cuda_stream))
+
+    def new_inputs(seed):
+        for i, (_, k) in enumerate(shapes):
+            xs[i].copy_(to_dev(oracle.fill_activations(seed + i, k)))
+
+    new_inputs(1)
+    call()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for seed in (10, 20, 30):
+        new_inputs(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [to_host(y).copy() for y in ys]
+        call()  # eager, with the K split and fresh epochs, between the replays
+        torch.cuda.synchronize()
+        for i in range(3):
+            assert rel_l2(got[i], to_host(ys[i])) < 2e-6, (seed, i)
+    aq = oracle.quantize_rows(to_host(xs[2]).reshape(1, -1))[0]
+    assert rel_l2(got[2], oracle.gemv(to_host(q8.untile(ws[2], *shapes[2])), aq, *shapes[2])) <= REL_L2_TOL
