@@ -5,7 +5,6 @@
 #include "q8_0_device.h"
 
 #include <cstring>
-#include <vector>
 
 namespace {
 
@@ -387,32 +386,43 @@ int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* co
 
 int nh_q8_0_gemv_tiled_group_f32(const void* const* host_W_tiled, const float* const* host_x, float* const* host_y, const float* const* host_residual, const int64_t* host_N,
 	const int64_t* host_K, int64_t count, void* stream) {
-	NH_REQUIRE(count >= 0 && count <= 4096, NH_ERR_ARGUMENT);
+	NH_REQUIRE(count >= 0, NH_ERR_ARGUMENT);
 	if (count == 0) {
 		return NH_OK;
 	}
 	NH_REQUIRE(host_W_tiled && host_x && host_y && host_N && host_K, NH_ERR_NULL_POINTER);
-	std::vector<nh::gemv_group_op> ops;
-	ops.reserve(static_cast<size_t>(count));
+	// everything is checked before the first launch, so a bad entry cannot leave half the list enqueued
+	bool any = false;
 	for (int64_t i = 0; i < count; ++i) {
 		NH_TRY(check_shape(host_N[i], 0, host_K[i], true));
 		if (host_N[i] == 0) {
 			continue;
 		}
-		const float* res = host_residual ? host_residual[i] : nullptr;
+		any = true;
 		NH_REQUIRE(host_y[i], NH_ERR_NULL_POINTER);
-		NH_REQUIRE(aligned16(host_y[i]) && aligned16(res), NH_ERR_ALIGNMENT);
+		NH_REQUIRE(aligned16(host_y[i]) && (!host_residual || aligned16(host_residual[i])), NH_ERR_ALIGNMENT);
 		if (host_K[i] > 0) {
 			NH_REQUIRE(host_W_tiled[i] && host_x[i], NH_ERR_NULL_POINTER);
 			NH_REQUIRE(aligned16(host_W_tiled[i]) && aligned16(host_x[i]), NH_ERR_ALIGNMENT);
 		}
-		ops.push_back({ host_W_tiled[i], host_x[i], host_y[i], res, host_N[i], host_K[i] });
 	}
-	if (ops.empty()) {
+	if (!any) {
 		return NH_OK;
 	}
 	NH_TRY(require_device());
-	return from_hip(nh::launch_gemv_independent(ops.data(), static_cast<int64_t>(ops.size()), as_stream(stream)));
+	constexpr int CHUNK = 64; // a multiple of the group size: chunk borders fall on group borders
+	nh::gemv_group_op ops[CHUNK];
+	int n = 0;
+	for (int64_t i = 0; i < count; ++i) {
+		if (host_N[i] > 0) {
+			ops[n++] = { host_W_tiled[i], host_x[i], host_y[i], host_residual ? host_residual[i] : nullptr, host_N[i], host_K[i] };
+		}
+		if (n == CHUNK || (i + 1 == count && n > 0)) {
+			NH_TRY(from_hip(nh::launch_gemv_independent(ops, n, as_stream(stream))));
+			n = 0;
+		}
+	}
+	return NH_OK;
 }
 
 int nh_q8_0_prepare(void) {

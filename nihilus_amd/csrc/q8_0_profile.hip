@@ -136,10 +136,14 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 		if (need < 0 || need > workspace_bytes) {
 			return NH_ERR_ARGUMENT;
 		}
-		if (op.M > 0 && op.N > 0 && (!op.W_tiled || !op.x || !op.y)) {
+		if (op.M > 0 && op.N > 0 && (!op.y || (op.K > 0 && (!op.W_tiled || !op.x)))) {
 			return NH_ERR_NULL_POINTER;
 		}
+		if (op.M > 0 && op.N > 0 && ((reinterpret_cast<uintptr_t>(op.W_tiled) | reinterpret_cast<uintptr_t>(op.x) | reinterpret_cast<uintptr_t>(op.y)) & 15u) != 0) {
+			return NH_ERR_ALIGNMENT;
+		}
 	}
+	constexpr int64_t MAX_RUN = 64; // M == 1 entries looked at together (a multiple of the group size)
 	const float* quantized_x = nullptr; // activation currently held in the workspace (M > 1 only)
 	int64_t quantized_m = -1, quantized_k = -1;
 	for (int64_t i = 0; i < count;) {
@@ -160,7 +164,7 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 			bool shared = true; // every entry of the run has the first one's x and K
 			while (i + g < count) {
 				const nh_q8_0_mul_mat_op& o = host_ops[i + g];
-				if (g >= 64 || o.M != 1 || o.N == 0 || o.ordered) { // 64: the hazard check is quadratic in the run length
+				if (g >= MAX_RUN || o.M != 1 || o.N == 0 || o.ordered) { // MAX_RUN: the hazard check is quadratic in the run length
 					break;
 				}
 				bool hazard = false;
@@ -189,19 +193,19 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 					return rc;
 				}
 			} else {
-				std::vector<const void*> w(static_cast<size_t>(g));
-				std::vector<const float*> x(static_cast<size_t>(g));
-				std::vector<float*> y(static_cast<size_t>(g));
-				std::vector<int64_t> n(static_cast<size_t>(g)), k(static_cast<size_t>(g));
+				const void* w[MAX_RUN];
+				const float* x[MAX_RUN];
+				float* y[MAX_RUN];
+				int64_t n[MAX_RUN], k[MAX_RUN];
 				for (int64_t e = 0; e < g; ++e) {
 					const nh_q8_0_mul_mat_op& o = host_ops[i + e];
-					w[static_cast<size_t>(e)]	= o.W_tiled;
-					x[static_cast<size_t>(e)]	= o.x;
-					y[static_cast<size_t>(e)]	= o.y;
-					n[static_cast<size_t>(e)]	= o.N;
-					k[static_cast<size_t>(e)]	= o.K;
+					w[e] = o.W_tiled;
+					x[e] = o.x;
+					y[e] = o.y;
+					n[e] = o.N;
+					k[e] = o.K;
 				}
-				const int rc = nh_q8_0_gemv_tiled_group_f32(w.data(), x.data(), y.data(), nullptr, n.data(), k.data(), g, stream);
+				const int rc = nh_q8_0_gemv_tiled_group_f32(w, x, y, nullptr, n, k, g, stream);
 				if (rc != NH_OK) {
 					return rc;
 				}

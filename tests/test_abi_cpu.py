@@ -71,6 +71,17 @@ def test_arguments_are_rejected_before_any_device_work():
     assert lib.nh_q8_0_mul_mat_batch(None, 3, None, 0, None) == -1
     ops = (_lib.MulMatOp * 1)(_lib.MulMatOp(bogus, bogus, bogus, 1, 32, 100, 0, 0))
     assert lib.nh_q8_0_mul_mat_batch(ops, 1, None, 0, None) == -3
+    ops = (_lib.MulMatOp * 1)(_lib.MulMatOp(bogus, bogus + 4, bogus, 1, 32, 128, 0, 0))
+    assert lib.nh_q8_0_mul_mat_batch(ops, 1, None, 0, None) == -2  # misaligned x: caught before the first launch
+    vp, i64 = C.c_void_p * 2, C.c_int64 * 2
+    w, x, y = vp(bogus, bogus), vp(bogus, bogus), vp(bogus, bogus)
+    assert lib.nh_q8_0_gemv_tiled_group_f32(w, x, y, None, i64(32, 32), i64(128, 100), 2, None) == -3
+    assert lib.nh_q8_0_gemv_tiled_group_f32(w, x, y, None, i64(32, 32), i64(128, 128), -1, None) == -6
+    assert lib.nh_q8_0_gemv_tiled_group_f32(w, None, y, None, i64(32, 32), i64(128, 128), 2, None) == -1
+    assert lib.nh_q8_0_gemv_tiled_group_f32(w, vp(bogus, None), y, None, i64(32, 32), i64(128, 128), 2, None) == -1
+    assert lib.nh_q8_0_gemv_tiled_group_f32(w, x, vp(bogus, bogus + 8), None, i64(32, 32), i64(128, 128), 2, None) == -2
+    assert lib.nh_q8_0_gemv_tiled_group_f32(w, x, y, vp(bogus, bogus + 4), i64(32, 32), i64(128, 128), 2, None) == -2
+    assert lib.nh_q8_0_gemv_tiled_group_f32(w, x, y, None, i64(0, 0), i64(128, 128), 2, None) == 0  # nothing to do
     # empty work is success without a device
     assert lib.nh_q8_0_quantize(None, None, 0, 32, None) == 0
     assert lib.nh_q8_0_gemm(None, None, None, 0, 0, 128, None) == 0
