@@ -202,9 +202,11 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 				norm->scale = rms_scale_workgroup(p, norm->red, norm->wave, lane, norm->K, norm->eps);
 				norm->ready = true;
 			}
-			// a use of the last slice register: the compiler has to wait for the slice here, which (issue order) covers the
-			// memory -> LDS loads; the LDS reads below may not move above this point
-			asm volatile("" ::"v"(xf[XF_LOADS - 1].w) : "memory");
+			// a use of the last slice register that a load fills (the ones past the slice hold constants): the compiler has
+			// to wait for the slice here, which (issue order) covers the memory -> LDS loads; the LDS reads below may not
+			// move above this point
+			constexpr int LAST_LOADED = cnt > 0 ? (cnt * 32 - 1) / 64 : 0;
+			asm volatile("" ::"v"(xf[LAST_LOADED].w) : "memory");
 #pragma unroll
 			for (int i = 0; i < XF_LOADS; ++i) {
 				const int v = lane + 64 * i;

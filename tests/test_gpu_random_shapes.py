@@ -38,6 +38,24 @@ def test_random_single_and_residual_mat_vecs(q8, oracle, seed):
         assert rel_l2(to_host(q8.gemv_residual_f32(wt, to_dev(x), to_dev(r), n, k)), want + r) <= REL_L2_TOL, (seed, case, n, k, "residual")
         xq = q8.quantize_row_q8_0(to_dev(x))
         assert rel_l2(to_host(q8.gemv(wt, xq, n, k, tiled=True)), want) <= REL_L2_TOL, (seed, case, n, k, "blocks in")
+        nw = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+        want_n = oracle.gemv(w, oracle.rms_norm_quantize_rows(x[None, :], nw, 1e-5)[0], n, k)
+        assert rel_l2(to_host(q8.gemv_f32(wt, to_dev(x), n, k, norm_weight=to_dev(nw), eps=1e-5)), want_n) <= REL_L2_TOL, (seed, case, n, k, "norm inside")
+
+
+def test_norm_inside_with_waves_of_unequal_group_counts(q8, oracle):
+    # K = 5120 is 40 groups: in an unsplit launch eight waves own three and eight own two, in the four-group kernel variant.
+    # The quantizer's wait for the activation slice must name a register that a load fills for every count
+    # (a wave with two groups has none in the upper half of the slice registers).
+    rng = np.random.default_rng(77)
+    for n, k in ((8192, 5120), (600, 5120), (3000, 2560 + 128)):
+        w = random_blocks(rng, n, k)
+        x = rng.standard_normal(k).astype(np.float32)
+        nw = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+        wt = q8.tile(to_dev(w), n, k)
+        want = oracle.gemv(w, oracle.rms_norm_quantize_rows(x[None, :], nw, 1e-5)[0], n, k)
+        for rep in range(3):
+            assert rel_l2(to_host(q8.gemv_f32(wt, to_dev(x), n, k, norm_weight=to_dev(nw), eps=1e-5)), want) <= REL_L2_TOL, (n, k, rep)
 
 
 @pytest.mark.parametrize("seed", range(8))
@@ -76,3 +94,27 @@ def test_random_small_m_mul_mat(q8, oracle, seed):
         want = _want(oracle, w, x, n, k)
         assert rel_l2(to_host(q8.mul_mat(wt, to_dev(x), n, k)), want) <= REL_L2_TOL, (seed, case, m, n, k)
         assert rel_l2(to_host(q8.mul_mat(wt, to_dev(x), n, k, residual=to_dev(r))), want + r) <= REL_L2_TOL, (seed, case, m, n, k, "residual")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_one_launch_ffn(q8, oracle, seed):
+    # the stages of the one-launch FFN against the checker: gate / up from the launch's own inspection copies, the down stage
+    # re-derived from them (so its activation quantize is checked bit for bit in effect), with and without norm and residual
+    rng = np.random.default_rng(4000 + seed)
+    n_ff = 128 * int(rng.choice([rng.integers(1, 9), rng.integers(9, 60)]))
+    k = 128 * int(rng.choice([rng.integers(1, 9), rng.integers(9, 48)]))
+    n_out = int(rng.choice([rng.integers(1, 100), rng.integers(100, 2500)]))
+    sg, sd = 1.0 / (58.0 * np.sqrt(k)), 1.0 / (58.0 * np.sqrt(n_ff))
+    wg, wu, wd = random_blocks(rng, n_ff, k, sg), random_blocks(rng, n_ff, k, sg), random_blocks(rng, n_out, n_ff, sd)
+    wg_t, wu_t, wd_t = (q8.tile(to_dev(w), r, c) for w, r, c in ((wg, n_ff, k), (wu, n_ff, k), (wd, n_out, n_ff)))
+    x = rng.standard_normal(k).astype(np.float32)
+    res = rng.standard_normal(n_out).astype(np.float32)
+    nw = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    for use_norm, use_res in ((False, False), (True, True)):
+        y = q8.ffn(wg_t, wu_t, wd_t, to_dev(x), n_ff, k, n_out, residual=to_dev(res) if use_res else None, norm_weight=to_dev(nw) if use_norm else None, eps=1e-5)
+        g, u = (to_host(t) for t in q8.debug_ffn_gate_up(n_ff))
+        xq = oracle.rms_norm_quantize_rows(x[None, :], nw, 1e-5)[0] if use_norm else oracle.quantize_rows(x[None, :])[0]
+        tag = (seed, n_ff, k, n_out, use_norm)
+        assert rel_l2(g, oracle.gemv(wg, xq, n_ff, k)) <= REL_L2_TOL and rel_l2(u, oracle.gemv(wu, xq, n_ff, k)) <= REL_L2_TOL, tag
+        want = oracle.gemv(wd, oracle.silu_mul_quantize_rows(g, u)[0], n_out, n_ff) + (res if use_res else 0)
+        assert rel_l2(to_host(y), want) <= REL_L2_TOL, tag
