@@ -1,7 +1,7 @@
 """GPU: seeded random shapes through every mat-vec / small-M entry point, each result against the CPU checker.
 
 The named tests pin the shapes of the benchmark configurations; this one walks the space between them (ragged row counts,
-K from one group to 120, every cut the planner can choose: row parts, K splits, chunked walks, grouped launches of mixed
+K from one group to 299, every cut the planner can choose: row parts, K splits, chunked walks, grouped launches of mixed
 shapes, 2- and 3-row forms, the MFMA streaming kernel from M = 4) so that a shape-dependent mistake in a path the named
 tests do not happen to take shows up here.  Seeds are fixed: a failure names its case and can be rerun.
 """
@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 def _shape(rng):
     n = int(rng.choice([rng.integers(1, 64), rng.integers(64, 700), rng.integers(700, 3000)]))
-    k = 128 * int(rng.choice([rng.integers(1, 5), rng.integers(5, 40), rng.integers(40, 121)]))
+    k = 128 * int(rng.choice([rng.integers(1, 5), rng.integers(5, 40), rng.integers(40, 121), rng.integers(121, 300)]))
     return n, k
 
 
@@ -118,3 +118,39 @@ def test_random_one_launch_ffn(q8, oracle, seed):
         assert rel_l2(g, oracle.gemv(wg, xq, n_ff, k)) <= REL_L2_TOL and rel_l2(u, oracle.gemv(wu, xq, n_ff, k)) <= REL_L2_TOL, tag
         want = oracle.gemv(wd, oracle.silu_mul_quantize_rows(g, u)[0], n_out, n_ff) + (res if use_res else 0)
         assert rel_l2(to_host(y), want) <= REL_L2_TOL, tag
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_prefill_path(q8, oracle, seed):
+    # quantizers bit for bit (blocks and tiled), then the mat-mat on the tile kernel's side of the routing (M > 64) and
+    # the raw-blocks twin, with ragged M and N
+    rng = np.random.default_rng(5000 + seed)
+    m = int(rng.choice([rng.integers(65, 130), rng.integers(130, 400)]))
+    n = int(rng.choice([rng.integers(1, 200), rng.integers(200, 2500)]))
+    k = 128 * int(rng.choice([rng.integers(1, 6), rng.integers(6, 33)]))
+    w = random_blocks(rng, n, k)
+    x = (rng.standard_normal((m, k)) * rng.choice([1e-3, 1.0, 300.0])).astype(np.float32)
+    tag = (seed, m, n, k)
+    aq_cpu = oracle.quantize_rows(x)
+    aq = q8.quantize_row_q8_0(to_dev(x))
+    assert np.array_equal(to_host(aq).reshape(m, -1), aq_cpu), tag
+    aq_t = q8.quantize_row_q8_0(to_dev(x), tiled=True)
+    assert np.array_equal(to_host(q8.untile(aq_t, m, k)).reshape(m, -1), aq_cpu), tag
+    nw = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    an_t = q8.rms_norm_quantize(to_dev(x), to_dev(nw), 1e-5, tiled=True)
+    assert np.array_equal(to_host(q8.untile(an_t, m, k)).reshape(m, -1), oracle.rms_norm_quantize_rows(x, nw, 1e-5)), tag
+    g, u = rng.standard_normal((m, k)).astype(np.float32) * 3, rng.standard_normal((m, k)).astype(np.float32)
+    as_t = q8.silu_mul_quantize(to_dev(g), to_dev(u), tiled=True)
+    assert np.array_equal(to_host(q8.untile(as_t, m, k)).reshape(m, -1), oracle.silu_mul_quantize_rows(g, u)), tag
+    want = oracle.gemm(w, aq_cpu, m, n, k, threads=4) if (k // 32) % 16 == 0 else oracle.gemm(w, aq_cpu, m, n, k)
+    wt = q8.tile(to_dev(w), n, k)
+    r = rng.standard_normal((m, n)).astype(np.float32)
+    assert rel_l2(to_host(q8.gemm(wt, aq_t, m, n, k, tiled=True)), want) <= REL_L2_TOL, tag
+    assert rel_l2(to_host(q8.gemm_residual(wt, aq_t, to_dev(r), m, n, k)), want + r) <= REL_L2_TOL, tag
+    assert rel_l2(to_host(q8.gemm(to_dev(w), aq, m, n, k, tiled=False)), want) <= REL_L2_TOL, tag
+    assert rel_l2(to_host(q8.mul_mat(wt, to_dev(x), n, k)), want) <= REL_L2_TOL, tag
+    # token rows out of the same matrix, some ids out of range
+    ids = rng.integers(-2, n + 2, size=37).astype(np.int32)
+    got = q8.get_rows(wt, to_dev(ids), n, k, tiled=True)
+    want_rows = oracle.get_rows(w, ids, n, k)[0]
+    assert np.array_equal(to_host(got), want_rows), tag
