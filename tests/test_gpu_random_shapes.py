@@ -154,3 +154,32 @@ def test_random_prefill_path(q8, oracle, seed):
     got = q8.get_rows(wt, to_dev(ids), n, k, tiled=True)
     want_rows = oracle.get_rows(w, ids, n, k)[0]
     assert np.array_equal(to_host(got), want_rows), tag
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_blocks_layout_and_block_sums(q8, oracle, seed):
+    # the reference's packed blocks as they come (K any multiple of 32): quantize, mat-vec, mat-mat, get_rows; and the int32
+    # block sums of all four kernel families, bit for bit
+    rng = np.random.default_rng(6000 + seed)
+    n = int(rng.choice([rng.integers(1, 40), rng.integers(40, 900)]))
+    k = 32 * int(rng.choice([rng.integers(1, 9), rng.integers(9, 200)]))
+    m = int(rng.choice([1, 2, 7, 33, 90]))
+    tag = (seed, m, n, k)
+    w = random_blocks(rng, n, k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    aq_cpu = oracle.quantize_rows(x)
+    aq = q8.quantize_row_q8_0(to_dev(x))
+    assert np.array_equal(to_host(aq).reshape(m, -1), aq_cpu), tag
+    want = oracle.gemm(w, aq_cpu, m, n, k)
+    wd = to_dev(w)
+    assert rel_l2(to_host(q8.gemv(wd, aq.reshape(m, -1)[0].contiguous(), n, k, tiled=False)), want[0]) <= REL_L2_TOL, tag
+    assert rel_l2(to_host(q8.gemm(wd, aq, m, n, k, tiled=False)), want) <= REL_L2_TOL, tag
+    sums = np.stack([oracle.block_sums_gemv(w, aq_cpu[i], n, k) for i in range(m)])
+    assert np.array_equal(to_host(q8.debug_block_sums(wd, aq.reshape(m, -1)[0].contiguous(), 1, n, k, path=0))[0], sums[0]), tag
+    assert np.array_equal(to_host(q8.debug_block_sums(wd, aq, m, n, k, path=1)), sums), tag
+    ids = rng.integers(0, n, size=11).astype(np.int32)
+    assert np.array_equal(to_host(q8.get_rows(wd, to_dev(ids), n, k, tiled=False)), oracle.get_rows(w, ids, n, k)[0]), tag
+    if k % 128 == 0:
+        wt = q8.tile(wd, n, k)
+        assert np.array_equal(to_host(q8.debug_block_sums(wt, aq.reshape(m, -1)[0].contiguous(), 1, n, k, path=2))[0], sums[0]), tag
+        assert np.array_equal(to_host(q8.debug_block_sums(wt, q8.tile(aq, m, k), m, n, k, path=3)), sums), tag
