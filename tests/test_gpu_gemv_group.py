@@ -130,3 +130,37 @@ def test_batch_runner_groups_independent_entries_only(q8, oracle):
     assert rel_l2(to_host(y_c), to_host(q8.gemv_f32(ws[0], xs[2], n, k))) < 2e-6
     # and the chain's first stage against the checker
     assert rel_l2(to_host(y_a), oracle.gemv(ws_host[0], oracle.quantize_rows(to_host(x0).reshape(1, k))[0], n, k)) <= REL_L2_TOL
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_batch_runner_random_dependency_patterns(q8, seed):
+    # random lists of M = 1 entries over a small pool of buffers, so that reads-after-writes, writes-after-reads and
+    # writes-after-writes occur in every position; the batch call must leave the pool exactly as one-by-one execution in
+    # list order does.  The shape is one whose single launch and grouped form do the same arithmetic in the same order
+    # (132 strips: no row split), so "exactly" means bit for bit however deep the chains get.
+    import torch
+
+    from nihilus_amd import _lib
+
+    lib = _lib.lib()
+    rng = np.random.default_rng(300 + seed)
+    d = 4224
+    hw = [random_blocks(rng, d, d, 1.0 / (58.0 * np.sqrt(d))) for _ in range(4)]  # about unit gain, so chains stay finite
+    ws = [q8.tile(to_dev(w), d, d) for w in hw]
+    pool0 = [q8.fill_activations(600 + i, d) for i in range(5)]
+    entries = []
+    for _ in range(14):
+        src, dst = rng.choice(5, size=2, replace=False)
+        entries.append((int(rng.integers(0, 4)), int(src), int(dst), int(rng.integers(0, 4) == 0)))
+    pool = [p.clone() for p in pool0]
+    ops = (_lib.MulMatOp * len(entries))()
+    for i, (wi, src, dst, ordered) in enumerate(entries):
+        ops[i] = _lib.MulMatOp(ws[wi].data_ptr(), pool[src].data_ptr(), pool[dst].data_ptr(), 1, d, d, 0, ordered)
+    dummy = torch.empty(256, dtype=torch.uint8, device="cuda")
+    _lib.check("nh_q8_0_mul_mat_batch", lib.nh_q8_0_mul_mat_batch(ops, len(entries), dummy.data_ptr(), dummy.numel(), torch.cuda.current_stream().cuda_stream))
+    ref2 = [p.clone() for p in pool0]  # one by one, in list order
+    for wi, src, dst, _ in entries:
+        ref2[dst].copy_(q8.gemv_f32(ws[wi], ref2[src], d, d))
+    for i in range(5):
+        a, b = to_host(pool[i]), to_host(ref2[i])
+        assert np.isfinite(b).all() and np.array_equal(a, b), (seed, i, entries)
