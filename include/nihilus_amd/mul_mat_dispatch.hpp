@@ -291,6 +291,29 @@ namespace nihilus {
 		}
 	};
 
+	// The key the reference implements on the CPU, <float, block_q8_0<half>, float> (cpu/avx_2.hpp:4854-5004): fp32 activations
+	// against Q8_0 weights WITHOUT quantizing the activations, both phases (eval_time: one row; prompt_eval_time: the output's
+	// runtime sequence length).  Not the path a model runs; a plain form that reads the weights once per activation row.
+	template<typename config_type, typename core_traits_type, processing_phases processing_phase>
+	struct kernel_dispatcher_impl<config_type, core_traits_type, device_types::gpu, 5, kernel_types::mul_mat, processing_phase, core_traits_type, float, block_q8_0<half>, float> {
+		using input_type01			   = typename core_traits_type::input_01_type;
+		static constexpr uint64_t ne00 = input_type01::get_array()[0]; // K
+		static constexpr uint64_t ne01 = input_type01::get_array()[1]; // N
+		static_assert(ne00 % 128 == 0, "the tiled weight layout needs K to be a multiple of 128");
+
+		static void impl(core_traits_type& output, const void* weight_tiled, const float* activation, void* stream = nullptr) {
+			const uint64_t rows = processing_phase == processing_phases::eval_time ? 1 : output.get_seq_length_dim();
+			if (rows == 0) {
+				return;
+			}
+			amd_detail::check<config_type>(nh_q8_0_mul_mat_f32_activations(weight_tiled, activation, output.template get_data<float>(), static_cast<int64_t>(rows), ne01, ne00, stream),
+				"mul_mat with fp32 activations");
+			if constexpr (config_type::synchronous) {
+				amd_detail::check<config_type>(nh_stream_sync(stream), "stream sync");
+			}
+		}
+	};
+
 	// get_rows (token embeddings), both phases: out[t][:] = dequantized row ids[t] of the embedding table.  The table
 	// operand holds the device copy of token_embd.weight, tiled (table_is_tiled) or as the packed blocks of the file.
 	// eval_time looks up one token, prompt_eval_time the output's runtime sequence length; both index by the id (the

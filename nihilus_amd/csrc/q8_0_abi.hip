@@ -425,6 +425,18 @@ int nh_q8_0_gemv_tiled_group_f32(const void* const* host_W_tiled, const float* c
 	return NH_OK;
 }
 
+int nh_q8_0_mul_mat_f32_activations(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* stream) {
+	NH_TRY(check_shape(M, N, K, true));
+	if (M == 0 || N == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(y && (K == 0 || (W_tiled && x)), NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(W_tiled) && aligned16(x) && aligned16(y), NH_ERR_ALIGNMENT);
+	NH_REQUIRE(M * N <= MAX_BLOCKS, NH_ERR_TOO_LARGE);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_mul_mat_f32act(W_tiled, x, y, M, N, K, as_stream(stream)));
+}
+
 int nh_q8_0_prepare(void) {
 	NH_TRY(require_device());
 	const hipError_t e = nh::prepare_gemv_scratch();

@@ -253,6 +253,10 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	int64_t K, int64_t n_out, hipStream_t s);
 hipError_t copy_ffn_gate_up(float* gate_out, float* up_out, int64_t n_ff, hipStream_t s);
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w = nullptr, float norm_eps = 0.0f);
+// fp32 activations [M][K] against tiled Q8_0 weights without quantizing the activations (the reference's <float, block_q8_0, float>
+// mul_mat, cpu/avx_2.hpp:4782-5004): y [M][N].  K == 0 gives zeros.
+hipError_t launch_mul_mat_f32act(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s);
+
 // Mat-vecs that share nothing (own activation row, K, N) as one launch, up to GEMV_GROUP_MAX of them; the caller vouches that
 // none of them reads or overwrites another's output.  launch_gemv_group takes matrices whose waves own at most four groups
 // (anything plan_gemv can cut that way); launch_gemv_independent takes any list and falls back to single launches for the rest.

@@ -285,6 +285,17 @@ def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: t
     return y
 
 
+def mul_mat_f32_activations(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int) -> torch.Tensor:
+    """fp32 activations [M, K] (or [K]) x tiled Q8_0 weight [N, K] -> fp32 [M, N] without quantizing the activations."""
+    w_tiled, x = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(x, torch.float32, "x")
+    x2 = x.reshape(1, -1) if x.dim() == 1 else x
+    if x2.shape[1] != k or w_tiled.numel() != tiled_bytes(n, k):
+        raise ValueError("operand sizes do not match m x n x k")
+    y = torch.empty((x2.shape[0], n), dtype=torch.float32, device=x.device)
+    _lib.check("nh_q8_0_mul_mat_f32_activations", _lib.lib().nh_q8_0_mul_mat_f32_activations(w_tiled.data_ptr(), x2.data_ptr(), y.data_ptr(), x2.shape[0], n, k, _stream()))
+    return y
+
+
 def debug_block_sums(w: torch.Tensor, aq: torch.Tensor, m: int, n: int, k: int, path: int) -> torch.Tensor:
     """int32 [m, n, k/32] block sums: path 0/1 = mat-vec / MFMA kernel on blocks, 2/3 = the same on the tiled layout."""
     sums = torch.full((m, n, k // QK), -(2**31), dtype=torch.int32, device=w.device)

@@ -70,6 +70,8 @@ _gemv_f64 = _sig(_o, "nho_gemv_q8_0_f64", None, _vp, _vp, _vp, _i64, _i64)
 _gemm = _sig(_o, "nho_gemm_q8_0", None, _vp, _vp, _vp, _i64, _i64, _i64)
 _a_gemm = _sig(_a, "nha_gemm_q8_0_mt", C.c_int, _vp, _vp, _vp, _i64, _i64, _i64, C.c_int, C.c_int)
 _a_time_gemv = _sig(_a, "nha_time_gemv", C.c_double, _vp, _i64, _vp, _vp, _i64, _i64, C.c_int, C.c_int, C.c_int)
+_mul_mat_f32 = _sig(_o, "nho_mul_mat_q8_f32", None, _vp, _vp, _vp, _i64, _i64, _i64, C.c_int)
+_mul_mat_f32_f64 = _sig(_o, "nho_mul_mat_q8_f32_f64", None, _vp, _vp, _vp, _i64, _i64, _i64)
 _fill_act = _sig(_o, "nho_fill_activations", None, C.c_uint64, _vp, _i64)
 _fill_w = _sig(_o, "nho_fill_weight_blocks", None, C.c_uint64, _vp, _i64, _i64)
 
@@ -257,6 +259,22 @@ def gemv_f64(w: np.ndarray, xq: np.ndarray, n: int, k: int) -> np.ndarray:
     w, xq = _u8(w), _u8(xq)
     y = np.empty(n, dtype=np.float64)
     _gemv_f64(_ptr(w), _ptr(xq), _ptr(y), n, k)
+    return y
+
+
+def mul_mat_f32_activations(w: np.ndarray, x: np.ndarray, n: int, k: int, prompt_order: bool = False) -> np.ndarray:
+    """fp32 activations [m, k] against Q8_0 weights, no activation quantize: y [m, n] in the eval_time leaf's summation
+    order, or the prompt_eval_time leaf's."""
+    w, x = _u8(w), _f32(x).reshape(-1, k)
+    y = np.empty((x.shape[0], n), dtype=np.float32)
+    _mul_mat_f32(_ptr(w), _ptr(x), _ptr(y), x.shape[0], n, k, 1 if prompt_order else 0)
+    return y
+
+
+def mul_mat_f32_activations_f64(w: np.ndarray, x: np.ndarray, n: int, k: int) -> np.ndarray:
+    w, x = _u8(w), _f32(x).reshape(-1, k)
+    y = np.empty((x.shape[0], n), dtype=np.float64)
+    _mul_mat_f32_f64(_ptr(w), _ptr(x), _ptr(y), x.shape[0], n, k)
     return y
 
 

@@ -35,6 +35,10 @@
  *                                        correctly rounded double-precision value, <= 2 ulp over a dense sweep of
  *                                        the whole clamped range plus the special points; silu against float64.
  *   nho_block_sum_i32                    int64 brute force; extreme blocks (+-127 -> +-516128).
+ *   nho_vec_dot_q8_f32 / nho_scalar_dot_q8_f32 / nho_mul_mat_q8_f32
+ *                                        (fp32 activations, no activation quantize) float64 evaluation, d == 1 with integer
+ *                                        activations gives exact integers, the two reference orders agree to rounding,
+ *                                        equality with dequantize-then-dot in float64.
  *   nho_vec_dot_* / gemv / gemm          float64 evaluation (<= ~1e-6 rel), d == 1 gives exact
  *                                        integers, tiny hand-checkable shapes, gemm == M gemvs.
  *   The reference holds no golden vector for quantize or dot (its tests only print tok/s), and its
@@ -574,6 +578,76 @@ void nho_gemm_q8_0(const void* w, const void* aq, float* c, int64_t m_rows, int6
  *                   g = (sum - 393210) / 65536 exactly in fp32
  *   weight block t: qs[j] = ((u16 * 255) >> 16) - 127  -> uniform over [-127,127];
  *                   d = fp16(|gauss| * 0.01f)                                                  */
+/* ---- fp32 activations against Q8_0 weights, no activation quantize (the one mul_mat with a body in the reference) ---- */
+
+/* cpu/avx_2.hpp:4798-4816 (one block: sum of x_i * float(q_i) in element order, then times the scale) summed block after
+ * block as :4834-4851 does for a row of whole blocks; the eval_time dispatcher calls it per output row (:4978-5004). */
+float nho_vec_dot_q8_f32(const float* x, const void* vw, int64_t n_blocks) {
+	const uint8_t* w = (const uint8_t*)vw;
+	float sum		 = 0.0f;
+	for (int64_t b = 0; b < n_blocks; ++b) {
+		const float scale = nho_fp16_to_fp32(blk_d(w, b));
+		const int8_t* qs  = blk_qs(w, b);
+		float s			  = 0.0f;
+		for (int i = 0; i < NHO_QK; ++i) {
+			s += x[b * NHO_QK + i] * (float)qs[i];
+		}
+		sum += s * scale;
+	}
+	return sum;
+}
+
+/* cpu/avx_2.hpp:4881-4900, the prompt_eval_time dispatcher's leaf: sum += x * (float(q) * scale), element after element. */
+float nho_scalar_dot_q8_f32(const float* x, const void* vw, int64_t n_blocks) {
+	const uint8_t* w = (const uint8_t*)vw;
+	float sum		 = 0.0f;
+	for (int64_t b = 0; b < n_blocks; ++b) {
+		const float scale = nho_fp16_to_fp32(blk_d(w, b));
+		const int8_t* qs  = blk_qs(w, b);
+		for (int i = 0; i < NHO_QK; ++i) {
+			sum += x[b * NHO_QK + i] * ((float)qs[i] * scale);
+		}
+	}
+	return sum;
+}
+
+double nho_dot_q8_f32_f64(const float* x, const void* vw, int64_t n_blocks) {
+	const uint8_t* w = (const uint8_t*)vw;
+	double sum		 = 0.0;
+	for (int64_t b = 0; b < n_blocks; ++b) {
+		const double scale = (double)nho_fp16_to_fp32(blk_d(w, b));
+		const int8_t* qs   = blk_qs(w, b);
+		double s		   = 0.0;
+		for (int i = 0; i < NHO_QK; ++i) {
+			s += (double)x[b * NHO_QK + i] * (double)qs[i];
+		}
+		sum += s * scale;
+	}
+	return sum;
+}
+
+/* y[m][n] (n fastest, :4934 / :4959): order 0 = the eval_time leaf for every row, 1 = the prompt_eval_time leaf. */
+void nho_mul_mat_q8_f32(const void* vw, const float* x, float* y, int64_t m_rows, int64_t n_rows, int64_t k, int order) {
+	const uint8_t* w = (const uint8_t*)vw;
+	const int64_t nb = k / NHO_QK;
+	for (int64_t m = 0; m < m_rows; ++m) {
+		for (int64_t n = 0; n < n_rows; ++n) {
+			const uint8_t* row = w + n * nb * NHO_BLOCK_BYTES;
+			y[m * n_rows + n]  = order ? nho_scalar_dot_q8_f32(x + m * k, row, nb) : nho_vec_dot_q8_f32(x + m * k, row, nb);
+		}
+	}
+}
+
+void nho_mul_mat_q8_f32_f64(const void* vw, const float* x, double* y, int64_t m_rows, int64_t n_rows, int64_t k) {
+	const uint8_t* w = (const uint8_t*)vw;
+	const int64_t nb = k / NHO_QK;
+	for (int64_t m = 0; m < m_rows; ++m) {
+		for (int64_t n = 0; n < n_rows; ++n) {
+			y[m * n_rows + n] = nho_dot_q8_f32_f64(x + m * k, w + n * nb * NHO_BLOCK_BYTES, nb);
+		}
+	}
+}
+
 static inline uint64_t nho_hash(uint64_t seed, uint64_t i) {
 	uint64_t z = seed + (i + 1) * 0x9E3779B97F4A7C15ull;
 	z		   = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;

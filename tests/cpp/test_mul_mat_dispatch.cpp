@@ -15,6 +15,7 @@ void nho_fill_weight_blocks(uint64_t seed, void* out, int64_t first_block, int64
 void nho_quantize_rows_q8_0(const float* x, void* y, int64_t m, int64_t k);
 void nho_gemm_q8_0(const void* w, const void* aq, float* c, int64_t m, int64_t n, int64_t k);
 int64_t nho_get_rows_q8_0(const void* w, const int32_t* ids, float* out, int64_t n_tokens, int64_t n_rows, int64_t k);
+void nho_mul_mat_q8_f32(const void* w, const float* x, float* y, int64_t m_rows, int64_t n_rows, int64_t k, int order);
 }
 
 using namespace nihilus;
@@ -146,6 +147,26 @@ int main(int argc, char** argv) {
 		thrown = std::strstr(e.what(), "null pointer") != nullptr;
 	}
 	REQUIRE(thrown);
+
+	// the key the reference implements on the CPU, <float, block_q8_0<half>, float>: fp32 activations, no activation quantize
+	{
+		using f32_eval	 = kernel_dispatcher_impl<test_config, k_mul_mat_op, device_types::gpu, 5, kernel_types::mul_mat, processing_phases::eval_time, k_mul_mat_op, float, block_q8_0<half>, float>;
+		using f32_prompt = kernel_dispatcher_impl<test_config, k_mul_mat_op, device_types::gpu, 5, kernel_types::mul_mat, processing_phases::prompt_eval_time, k_mul_mat_op, float, block_q8_0<half>,
+			float>;
+		std::vector<float> want_f(M * N), got_f(M * N);
+		nho_mul_mat_q8_f32(w.data(), x.data(), want_f.data(), 1, N, K, 0); // the eval_time leaf's order
+		f32_eval::impl(op, d_tiled, static_cast<const float*>(d_x));
+		REQUIRE(nh_memcpy_d2h(got_f.data(), d_y, N * 4, nullptr) == NH_OK && nh_stream_sync(nullptr) == NH_OK);
+		const double e3 = rel_l2(std::vector<float>(got_f.begin(), got_f.begin() + N), std::vector<float>(want_f.begin(), want_f.begin() + N));
+		nho_mul_mat_q8_f32(w.data(), x.data(), want_f.data(), M, N, K, 1); // the prompt_eval_time leaf's
+		op.get_seq_length_dim() = M;
+		f32_prompt::impl(op, d_tiled, static_cast<const float*>(d_x));
+		REQUIRE(nh_memcpy_d2h(got_f.data(), d_y, M * N * 4, nullptr) == NH_OK && nh_stream_sync(nullptr) == NH_OK);
+		const double e4 = rel_l2(got_f, want_f);
+		std::printf("fp32 activations rel L2 %.3e (eval) %.3e (prompt)\n", e3, e4);
+		REQUIRE(e3 <= 1e-4 && e4 <= 1e-4);
+		op.get_seq_length_dim() = 0;
+	}
 
 	// token embeddings: bit-exact, both phases, both table layouts; eval_time must honour the id
 	{
