@@ -196,7 +196,7 @@ int nh_q8_0_gemm_tiled_residual(const void* W_tiled, const void* Aq_tiled, const
 /* Scratch the fused call needs for the quantized activations (device bytes, 256-byte aligned by the caller);
  * 0 for M <= 3, where the quantize happens inside the mat-vec kernel and workspace may be NULL. */
 int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K);
-/* quantize(x) then GEMV (M == 1; M = 2, 3: the same kernel with one dot product per row) or GEMM (M > 3) against a tiled weight: the whole
+/* quantize(x) then GEMV (M == 1; M = 2, 3, and M = 4, 5 on matrices up to 40 MB: the same kernel with one dot product per row) or GEMM (larger M) against a tiled weight: the whole
  * rms_norm-output -> projection step of core_traits.hpp:575-594 / :976-989 as one call. */
 int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 /* The same with the add node behind the projection folded in: y = mul_mat(W, x) + residual (fp32 [M][N], may be y itself),

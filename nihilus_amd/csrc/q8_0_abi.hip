@@ -540,7 +540,7 @@ static int mul_mat_common(const void* W_tiled, const float* x, const float* resi
 	if (M == 1) { // quantize fused into the mat-vec: the workspace stays unused
 		return residual ? nh_q8_0_gemv_tiled_residual_f32(W_tiled, x, residual, y, N, K, stream) : nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream);
 	}
-	if (M <= nh::GEMV_ROWS_MAX && K > 0) { // a few rows: the same streaming kernel with M dot products per weight tile
+	if (nh::gemv_rows_suits(M, N, K) && K > 0) { // a few rows: the same streaming kernel with M dot products per weight tile
 		NH_REQUIRE(W_tiled && y, NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(W_tiled) && aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
 		NH_TRY(require_device());

@@ -213,9 +213,9 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 			i += g;
 			continue;
 		}
-		if (op.M <= nh::GEMV_ROWS_MAX) {
-			// two or three rows: still the mat-vec kernel (one dot product per row), quantize inside, no workspace
-			const int rc = nh_q8_0_mul_mat(op.W_tiled, op.x, op.y, op.M, op.N, op.K, nullptr, 0, stream);
+		if (nh::gemv_rows_suits(op.M, op.N, op.K)) {
+			// a few rows: still the mat-vec kernel (one dot product per row), quantize inside, the workspace stays unused
+			const int rc = nh_q8_0_mul_mat(op.W_tiled, op.x, op.y, op.M, op.N, op.K, workspace, workspace_bytes, stream);
 			if (rc != NH_OK) {
 				return rc;
 			}

@@ -93,10 +93,11 @@ def test_mul_mat_fused(q8, oracle):
 @pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (14336, 4096), (33, 128), (100, 1024), (8192, 28672), (1024, 8192), (40000, 8192), (64, 128 * 70)])
 def test_mul_mat_few_rows(q8, oracle, n, k):
     # 2 or 3 activation rows: the streaming mat-vec with one dot product per row and weight tile, quantize inside the kernel
-    # (unsplit, K split over workgroups, chunked walk, ragged N); no workspace is needed there.  4 rows: the MFMA kernel.
+    # (unsplit, K split over workgroups, chunked walk, ragged N); no workspace is needed there.  4 and 5 rows: the same kernel on
+    # matrices up to 40 MB, quantize + the MFMA kernel on larger ones.  6 rows: the MFMA kernel.
     w = oracle.fill_weights(n + k, n, k)
     wt = q8.tile(to_dev(w), n, k)
-    for m in (2, 3, 4):
+    for m in (2, 3, 4, 5, 6):
         assert (q8._lib.lib().nh_q8_0_mul_mat_workspace_bytes(m, k) == 0) == (m <= 3)
         x = oracle.fill_activations(m + n, m * k).reshape(m, k)
         if m == 3:
