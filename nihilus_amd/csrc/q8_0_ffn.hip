@@ -62,8 +62,8 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 		__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1];
 		gemv_norm norm_state;
 		gemv_norm* norm = nullptr;
-		if constexpr (NORM) { // eight waves per matrix here: the slices are not the sixteen runs of the fixed order, so the scale comes first
-			gemv_norm_begin(norm_state, a.x, a.norm_w, xs_w[NORM ? wave : 0], norm_red, a.norm_eps, a.groups_p * GROUP_K, lane, wave, false);
+		if constexpr (NORM) { // the row's scale first
+			gemv_norm_begin(norm_state, a.x, a.norm_w, xs_w[NORM ? wave : 0], norm_red, a.norm_eps, a.groups_p * GROUP_K, lane, wave);
 			norm = &norm_state;
 		}
 		const int matrix	   = wave >> 3;

@@ -142,8 +142,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	float acc			   = 0.0f;
 	gemv_norm norm_state;
 	gemv_norm* norm = nullptr;
-	if constexpr (NORM) { // RMS norm * weight in front of the quantizer; an unsplit, single-chunk launch takes the sum from its slices
-		gemv_norm_begin(norm_state, static_cast<const float*>(xin), norm_w, xs_w[NORM ? wave : 0], norm_red, norm_eps, groups * GROUP_K, lane, wave, !LOOP && splits == 1);
+	if constexpr (NORM) { // RMS norm * weight in front of the quantizer: the row's scale first
+		gemv_norm_begin(norm_state, static_cast<const float*>(xin), norm_w, xs_w[NORM ? wave : 0], norm_red, norm_eps, groups * GROUP_K, lane, wave);
 		norm = &norm_state;
 	}
 	if constexpr (!LOOP) {

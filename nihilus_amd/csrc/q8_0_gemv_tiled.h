@@ -33,37 +33,25 @@ enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2 };
 constexpr int PUBLISHED_SPIN_LIMIT = 1 << 20;
 constexpr int PUBLISHED_WORDS	   = 9; // per block: quant dwords 0..7, then the scale
 
-// RMS norm * weight in front of the quantizer (X_F32 only).  The row's scale needs every element.  The fixed order
-// of the sum of squares (rms_run_* in q8_0_device.h) cuts the row into 16 runs exactly as an unsplit launch cuts K over
-// its 16 waves, so in that case the wave's activation slice, which it loads anyway, IS its share of the sum: no extra
-// load, one workgroup barrier while the weights are in flight (`from_slice`).  When K is split over workgroups or
-// walked in several chunks the slices do not cover the row, and the kernel works the scale out first from the row
-// itself (`ready`).  Loads return in issue order, so what the staging needs (the slice and its norm weights) is
-// requested BEFORE the weight stream: a load issued after it would only come back behind it.  The norm weights go
-// from memory straight into LDS (no destination registers: the kernel stays at two workgroups per CU).
+// RMS norm * weight in front of the quantizer (X_F32 only).  The row's scale needs every element, so the workgroup works it
+// out first, from the row itself (16 KB at K = 4096, served by cache for all but the first workgroups; fixed order of the sum of
+// squares: rms_run_* in q8_0_device.h; one workgroup barrier), before its weight loads go out.  Taking the sum from the waves'
+// own activation slices instead -- they are loaded anyway, and an unsplit launch cuts K over its 16 waves exactly as the
+// fixed order cuts the row -- saves that read but puts the barrier behind the slice loads, with the weight stream already
+// queued around them: measured 3-4 % slower ([14336 x 4096] 12.4 against 11.9 us), and it was the more fragile form.
+// Loads return in issue order, so what the staging needs (the slice and its norm weights) is requested BEFORE the weight
+// stream: a load issued after it would only come back behind it.  The norm weights go from memory straight into LDS (no
+// destination registers: the kernel stays at two workgroups per CU).
 struct gemv_norm {
 	const float* w; // norm weight, fp32 [K]
 	float4* xs_w; // this wave's LDS slice for the norm weights of its activation slice (TILES * 32 float4)
-	float* red; // 16 floats of LDS
-	float eps;
-	float scale;
-	int K;
-	int wave;
-	bool ready; // scale holds the row's 1 / rms
+	float scale; // the row's 1 / rms
 };
-__device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, const float* w, float4* xs_w, float* red, float eps, int K, int lane, int wave, bool from_slice) {
+// red: 16 floats of LDS.  Contains a workgroup barrier: every thread of the workgroup must call it.
+__device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, const float* w, float4* xs_w, float* red, float eps, int K, int lane, int wave) {
 	n.w		= w;
 	n.xs_w	= xs_w;
-	n.red	= red;
-	n.eps	= eps;
-	n.K		= K;
-	n.wave	= wave;
-	n.scale = 0.0f;
-	n.ready = false;
-	if (!from_slice) {
-		n.scale = rms_scale_workgroup(rms_run_sumsq(x, K / GROUP_K, wave, lane), red, wave, lane, K, eps);
-		n.ready = true;
-	}
+	n.scale = rms_scale_workgroup(rms_run_sumsq(x, K / GROUP_K, wave, lane), red, wave, lane, K, eps);
 }
 
 //
@@ -193,15 +181,6 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	// ---- 3. stage the activation slice in LDS: quants 16-byte aligned per half block, scales as fp32 ----
 	if constexpr (XF32) {
 		if constexpr (NORM) {
-			if (!norm->ready) { // the slice is this wave's run of the row: reduce over the workgroup (one barrier, weights in flight)
-				float p = 0.0f;
-#pragma unroll
-				for (int i = 0; i < XF_LOADS; ++i) {
-					p = sumsq_fold(p, xf[i]); // lanes past the slice hold zeros, which leave p unchanged
-				}
-				norm->scale = rms_scale_workgroup(p, norm->red, norm->wave, lane, norm->K, norm->eps);
-				norm->ready = true;
-			}
 			// a use of the last slice register that a load fills (the ones past the slice hold constants): the compiler has
 			// to wait for the slice here, which (issue order) covers the memory -> LDS loads; the LDS reads below may not
 			// move above this point
