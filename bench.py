@@ -64,7 +64,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
     ap.add_argument("--calibration-copies", type=int, default=0, help="run this many plain 64 MiB device copies first (a known-size kernel to scale hardware byte counters by)")
-    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover", "llama70b"], default="ffn_decode",
+    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover", "llama70b", "f32act"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
     ap.add_argument("--ffn-mode", choices=["group", "two", "fused"], default="group",
@@ -397,6 +397,40 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                 "higher_is_better": True, "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate", "data": "synthetic",
                 "config": {"workload": "nh_q8_0_mul_mat, fp32 activations [M x K] x Q8_0 W at the 70B shapes, M in {1, 4, 16, 64}, activation quantize included, "
                            "weight sets rotated over > 1 GB (lm_head: one 1.1 GB matrix)"}, "rows": rows}
+
+    if kind == "f32act":
+        # fp32 activations against Q8_0 weights without activation quantize (the reference's <float, block_q8_0, float> mul_mat), one
+        # activation row, the FFN decode shapes; 8 weight sets per shape rotated so that HBM is what is read
+        shapes = [(14336, K), (4096, 14336)]
+        rows = []
+        tot_bytes, tot_wall, dom = 0, 0.0, None
+        for si, (n, k) in enumerate(shapes):
+            wsets = [q8_0.tile(q8_0.fill_weight_blocks(20 + 8 * si + c, n, k), n, k) for c in range(8)]
+            xv = q8_0.fill_activations(5 + si, k)
+            yv = torch.empty(n, dtype=torch.float32, device=x.device)
+            nbytes = n * (k // 32) * 34 + 4 * k + 4 * n
+            it = [0]
+
+            def fn():
+                it[0] += 1
+                _lib.check("nh_q8_0_mul_mat_f32_activations", lib.nh_q8_0_mul_mat_f32_activations(wsets[it[0] % 8].data_ptr(), xv.data_ptr(), yv.data_ptr(), 1, n, k, stream))
+
+            wall, ksec, cnt = timed(1, fn, 1)
+            rows.append({"N": n, "K": k, "bytes_per_launch": nbytes, "avg_launch_us": round(ksec * 1e6, 3), "GBs": round(nbytes / ksec / 1e9, 1),
+                         "frac": round(nbytes / ksec / 1e9 / HBM_PEAK_GBS, 4), "wall_us": round(wall * 1e6, 3), "launches_timed": cnt, "outputs_finite": bool(torch.isfinite(yv).all().item())})
+            tot_bytes += nbytes
+            tot_wall += wall
+            if dom is None:
+                dom = (nbytes, ksec, cnt)
+            del wsets
+        ach = dom[0] / dom[1] / 1e9
+        return {
+            "metric": "Q8_0 weight x fp32 activation mat-vec GB/s", "value": round(tot_bytes / tot_wall / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(tot_wall * 1e3, 6), "higher_is_better": True, "dtype": "int8 -> fp32, fp32 multiply-accumulate", "data": "synthetic",
+            "config": {"workload": "fp32-activation mat-vec (no activation quantize), M=1, Q8_0 W [14336x4096] and [4096x14336], one launch each per step", "shapes": rows},
+            "roofline": {"bound": "hbm", "kernel": "nh::mul_mat_f32act_kernel ([14336x4096])", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": dom[0], "avg_launch_us": round(dom[1] * 1e6, 3), "launches_timed": dom[2]},
+        }
 
     if kind == "get_rows":
         n_rows = 128256  # LLaMA-3 vocabulary; token_embd.weight [4096 x 128256] Q8_0 = 558 MB, rows picked at random

@@ -14,8 +14,10 @@ namespace nh {
 
 constexpr int F32ACT_WAVES = 16;
 
-__global__ __launch_bounds__(F32ACT_WAVES * 64) void mul_mat_f32act_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int N, int groups) {
-	__shared__ __align__(16) float xs[F32ACT_WAVES][GROUP_K];
+// GC groups per step: every load of the step (weights, scales, activation slice) is issued before the first one is waited
+// for, so a wave has GC * 4 KiB in flight; a group past the wave's range repeats the last one (a cache hit, not used).
+template<int GC> __global__ __launch_bounds__(F32ACT_WAVES * 64, GC <= 2 ? 8 : 4) void mul_mat_f32act_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int N, int groups) {
+	__shared__ __align__(16) float xs[F32ACT_WAVES][GC][GROUP_K];
 	__shared__ float red[F32ACT_WAVES][64];
 	const int tid	= threadIdx.x;
 	const int lane	= tid & 63;
@@ -26,38 +28,58 @@ __global__ __launch_bounds__(F32ACT_WAVES * 64) void mul_mat_f32act_kernel(const
 	const int r		= lane & 31;
 	int g0, g1;
 	wave_k_range(groups, 0, 0, F32ACT_WAVES, wave, g0, g1);
-	const float* xrow = x + m * static_cast<int64_t>(groups) * GROUP_K;
-	float acc		  = 0.0f;
-	for (int g = g0; g < g1; ++g) {
-		const uint8_t* macro = W + macro_offset(strip, g, groups);
-		v4i q[GROUP_BLOCKS];
+	const float* xrow	   = x + m * static_cast<int64_t>(groups) * GROUP_K;
+	const uint8_t* w_strip = W + macro_offset(strip, 0, groups);
+	float acc			   = 0.0f;
+	// GC == 2 is launched only where a wave has at most two groups: one step, no loop state
+	for (int g = g0; g < g1; g += (GC == 2 ? (1 << 30) : GC)) {
+		v4i q[GC][GROUP_BLOCKS];
+		v2u dd[GC];
+		// the activation slices go from memory straight into LDS, two groups (64 lanes x 16 bytes) per transfer, no registers
 #pragma unroll
-		for (int j = 0; j < GROUP_BLOCKS; ++j) {
-			q[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+		for (int c = 0; c < GC; c += 2) {
+			const int gg = min(g + c + half, g1 - 1);
+			load_global_to_lds_b128(xrow + static_cast<int64_t>(gg) * GROUP_K + 4 * r, &xs[wave][c][0]);
 		}
-		const v2u dd = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
-		if (lane < GROUP_K / 4) {
-			*reinterpret_cast<float4*>(&xs[wave][4 * lane]) = *reinterpret_cast<const float4*>(xrow + static_cast<int64_t>(g) * GROUP_K + 4 * lane);
+		asm volatile("" ::: "memory"); // the loads below are issued after the transfers
+#pragma unroll
+		for (int c = 0; c < GC; ++c) {
+			dd[c] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(w_strip + static_cast<int64_t>(min(g + c, g1 - 1)) * MACRO_BYTES + MACRO_D_OFFSET + 8 * r));
 		}
-		__builtin_amdgcn_wave_barrier(); // wave-local: the same wave wrote and reads
-		const float dw[GROUP_BLOCKS] = { half_bits_to_float(static_cast<uint16_t>(dd.x & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd.x >> 16)),
-			half_bits_to_float(static_cast<uint16_t>(dd.y & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd.y >> 16)) };
 #pragma unroll
-		for (int j = 0; j < GROUP_BLOCKS; ++j) {
-			const float* xb = &xs[wave][j * QK + 16 * half];
-			float s			= 0.0f;
+		for (int c = 0; c < GC; ++c) {
+			const uint8_t* macro = w_strip + static_cast<int64_t>(min(g + c, g1 - 1)) * MACRO_BYTES;
 #pragma unroll
-			for (int c = 0; c < 4; ++c) {
-				const float4 xv = *reinterpret_cast<const float4*>(xb + 4 * c);
-				const int word	= q[j][c];
-				s				= fmaf(xv.x, static_cast<float>(static_cast<int8_t>(word & 0xFF)), s);
-				s				= fmaf(xv.y, static_cast<float>(static_cast<int8_t>((word >> 8) & 0xFF)), s);
-				s				= fmaf(xv.z, static_cast<float>(static_cast<int8_t>((word >> 16) & 0xFF)), s);
-				s				= fmaf(xv.w, static_cast<float>(static_cast<int8_t>((word >> 24) & 0xFF)), s);
+			for (int j = 0; j < GROUP_BLOCKS; ++j) {
+				q[c][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
 			}
-			acc = fmaf(s, dw[j], acc);
 		}
-		__builtin_amdgcn_wave_barrier(); // the next group overwrites this wave's slice
+		// loads complete in issue order: once the first scale load (issued after the transfers) is there, so are the slices; the
+		// LDS reads below may not move above this point
+		asm volatile("" ::"v"(dd[0].x) : "memory");
+#pragma unroll
+		for (int c = 0; c < GC; ++c) {
+			if (c == 0 || g + c < g1) {
+				const float dw[GROUP_BLOCKS] = { half_bits_to_float(static_cast<uint16_t>(dd[c].x & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[c].x >> 16)),
+					half_bits_to_float(static_cast<uint16_t>(dd[c].y & 0xFFFFu)), half_bits_to_float(static_cast<uint16_t>(dd[c].y >> 16)) };
+#pragma unroll
+				for (int j = 0; j < GROUP_BLOCKS; ++j) {
+					const float* xb = &xs[wave][c][j * QK + 16 * half];
+					float s			= 0.0f;
+#pragma unroll
+					for (int k = 0; k < 4; ++k) {
+						const float4 xv = *reinterpret_cast<const float4*>(xb + 4 * k);
+						const int word	= q[c][j][k];
+						s				= fmaf(xv.x, static_cast<float>(static_cast<int8_t>(word & 0xFF)), s);
+						s				= fmaf(xv.y, static_cast<float>(static_cast<int8_t>((word >> 8) & 0xFF)), s);
+						s				= fmaf(xv.z, static_cast<float>(static_cast<int8_t>((word >> 16) & 0xFF)), s);
+						s				= fmaf(xv.w, static_cast<float>(static_cast<int8_t>((word >> 24) & 0xFF)), s);
+					}
+					acc = fmaf(s, dw[j], acc);
+				}
+			}
+		}
+		asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this step's LDS reads are done before the next step's transfers overwrite the slices
 	}
 	red[wave][lane] = acc;
 	__syncthreads();
@@ -81,9 +103,12 @@ hipError_t launch_mul_mat_f32act(const void* W_tiled, const float* x, float* y, 
 	}
 	const int strips = static_cast<int>((N + STRIP_ROWS - 1) / STRIP_ROWS);
 	// the grid's second dimension holds at most 65535 rows: walk M in slabs
+	// a wave's share of K is groups / 16: two groups per step cover the 4096-wide projections in one step at two workgroups per CU,
+	// longer rows take four per step
+	const auto kernel = K / GROUP_K <= 2 * F32ACT_WAVES ? mul_mat_f32act_kernel<2> : mul_mat_f32act_kernel<4>;
 	for (int64_t m0 = 0; m0 < M; m0 += 65535) {
 		const int64_t rows = M - m0 < 65535 ? M - m0 : 65535;
-		const hipError_t e = launch_kernel(KIND_GEMV, mul_mat_f32act_kernel, dim3(static_cast<unsigned>(strips), static_cast<unsigned>(rows)), dim3(F32ACT_WAVES * 64), 0, s,
+		const hipError_t e = launch_kernel(KIND_GEMV, kernel, dim3(static_cast<unsigned>(strips), static_cast<unsigned>(rows)), dim3(F32ACT_WAVES * 64), 0, s,
 			static_cast<const uint8_t*>(W_tiled), x + m0 * K, y + m0 * N, static_cast<int>(N), static_cast<int>(K / GROUP_K));
 		if (e != hipSuccess) {
 			return e;
