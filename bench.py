@@ -633,6 +633,9 @@ def cpu_baseline(budget_s: float) -> dict:
     t_d = O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, threads, passes, pin=False)
     sec = 2 * t_g + t_d
     nbytes = 2 * cpu_gemv_bytes(GATE_N, HIDDEN) + cpu_gemv_bytes(HIDDEN, FFN)
+    # the same step on one thread (a few passes: ~10 ms each)
+    one_passes = int(max(2, min(passes, 2.0 / max(sec * threads, 1e-6))))  # about two seconds
+    sec_1 = 2 * O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, 1, 2 * one_passes, pin=False) + O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, 1, one_passes, pin=False)
     model = ""
     try:
         with open("/proc/cpuinfo") as f:
@@ -651,6 +654,7 @@ def cpu_baseline(budget_s: float) -> dict:
         f"AVX2/FMA/F16C restatement of the reference arithmetic, {threads} threads, rows claimed through an atomic chunk counter",
         "cpu_model": model,
         "ms_per_step": round(sec * 1e3, 3),
+        "single_thread": {"value": round(nbytes / sec_1 / 1e9, 2), "unit": "GB/s", "cores": 1, "ms_per_step": round(sec_1 * 1e3, 3), "passes": one_passes},
     }
 
 
