@@ -8,7 +8,7 @@
 // to fp32 and multiplies in fp32; a lane holds half a block (16 quants) of one weight row and reads the matching 16 activations
 // as LDS broadcasts.  One workgroup per (strip, activation row): M rows read the weights M times, which is what the reference's
 // loop does too.
-#include "q8_0_device.h"
+#include "q8_0_gemv_tiled.h"
 
 namespace nh {
 
@@ -16,18 +16,23 @@ constexpr int F32ACT_WAVES = 16;
 
 // GC groups per step: every load of the step (weights, scales, activation slice) is issued before the first one is waited
 // for, so a wave has GC * 4 KiB in flight; a group past the wave's range repeats the last one (a cache hit, not used).
-template<int GC> __global__ __launch_bounds__(F32ACT_WAVES * 64, GC <= 2 ? 8 : 4) void mul_mat_f32act_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int N, int groups) {
+template<int GC> __global__ __launch_bounds__(F32ACT_WAVES * 64, GC <= 2 ? 8 : 4) void mul_mat_f32act_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int N, int groups, int split_shift,
+	uint64_t* __restrict__ tagged, unsigned epoch) {
 	__shared__ __align__(16) float xs[F32ACT_WAVES][GC][GROUP_K];
 	__shared__ float red[F32ACT_WAVES][64];
 	const int tid	= threadIdx.x;
 	const int lane	= tid & 63;
 	const int wave	= __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int strip = static_cast<int>(blockIdx.x);
-	const int64_t m = blockIdx.y;
+	// split_shift > 0 (one activation row only): 1 << split_shift workgroups share a strip's K range and hand their partial
+	// sums over as the mat-vec does
+	const int splits = 1 << split_shift;
+	const int strip	 = static_cast<int>(blockIdx.x >> split_shift);
+	const int split	 = static_cast<int>(blockIdx.x) & (splits - 1);
+	const int64_t m	 = blockIdx.y;
 	const int half	= lane >> 5;
 	const int r		= lane & 31;
 	int g0, g1;
-	wave_k_range(groups, 0, 0, F32ACT_WAVES, wave, g0, g1);
+	wave_k_range(groups, split_shift, split, F32ACT_WAVES, wave, g0, g1);
 	const float* xrow	   = x + m * static_cast<int64_t>(groups) * GROUP_K;
 	const uint8_t* w_strip = W + macro_offset(strip, 0, groups);
 	float acc			   = 0.0f;
@@ -90,7 +95,9 @@ template<int GC> __global__ __launch_bounds__(F32ACT_WAVES * 64, GC <= 2 ? 8 : 4
 			total += red[w][tid] + red[w][32 + tid];
 		}
 		const int row = strip * STRIP_ROWS + tid;
-		if (row < N) {
+		if (splits > 1) {
+			split_k_finish(tagged, epoch, strip, splits, split, tid, total, y, row, N, nullptr);
+		} else if (row < N) {
 			y[m * N + row] = total;
 		}
 	}
@@ -102,14 +109,31 @@ hipError_t launch_mul_mat_f32act(const void* W_tiled, const float* x, float* y, 
 		return hipSuccess;
 	}
 	const int strips = static_cast<int>((N + STRIP_ROWS - 1) / STRIP_ROWS);
+	const int groups = static_cast<int>(K / GROUP_K);
+	// One row: K goes over several workgroups per strip where the mat-vec's plan says so (long rows, few strips), except on a
+	// capturing stream (the hand-off's epoch would be the same in every replay).
+	int shift		   = 0;
+	gemv_scratch sc;
+	if (M == 1 && !stream_is_capturing(s)) {
+		const gemv_plan p = plan_gemv(strips, K);
+		if (p.splits > 1) {
+			while ((1 << shift) < p.splits) {
+				++shift;
+			}
+			const hipError_t e = get_gemv_scratch(&sc, true);
+			if (e != hipSuccess) {
+				return e;
+			}
+		}
+	}
+	// two groups per step where a wave owns at most two (one step, two workgroups per CU), else four per step
+	const int per_split = (groups + (1 << shift) - 1) >> shift; // the longest K range of a workgroup, in groups
+	const auto kernel	= (per_split + F32ACT_WAVES - 1) / F32ACT_WAVES <= 2 ? mul_mat_f32act_kernel<2> : mul_mat_f32act_kernel<4>;
 	// the grid's second dimension holds at most 65535 rows: walk M in slabs
-	// a wave's share of K is groups / 16: two groups per step cover the 4096-wide projections in one step at two workgroups per CU,
-	// longer rows take four per step
-	const auto kernel = K / GROUP_K <= 2 * F32ACT_WAVES ? mul_mat_f32act_kernel<2> : mul_mat_f32act_kernel<4>;
 	for (int64_t m0 = 0; m0 < M; m0 += 65535) {
 		const int64_t rows = M - m0 < 65535 ? M - m0 : 65535;
-		const hipError_t e = launch_kernel(KIND_GEMV, kernel, dim3(static_cast<unsigned>(strips), static_cast<unsigned>(rows)), dim3(F32ACT_WAVES * 64), 0, s,
-			static_cast<const uint8_t*>(W_tiled), x + m0 * K, y + m0 * N, static_cast<int>(N), static_cast<int>(K / GROUP_K));
+		const hipError_t e = launch_kernel(KIND_GEMV, kernel, dim3(static_cast<unsigned>(strips) << shift, static_cast<unsigned>(rows)), dim3(F32ACT_WAVES * 64), 0, s,
+			static_cast<const uint8_t*>(W_tiled), x + m0 * K, y + m0 * N, static_cast<int>(N), groups, shift, sc.tagged, sc.epoch);
 		if (e != hipSuccess) {
 			return e;
 		}
