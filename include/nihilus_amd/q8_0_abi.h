@@ -207,7 +207,9 @@ int nh_q8_0_mul_mat_residual(const void* W_tiled, const float* x, const float* r
 /* fp32 activations against Q8_0 weights WITHOUT quantizing the activations: y[m][n] = sum_b f32(d_w) * sum_i x[m][32b+i] * q_w[i],
  * all in fp32.  The mul_mat the reference implements for the key <float, block_q8_0<half>, float> (leaf vec_dot_q8_f32,
  * cpu/avx_2.hpp:4782-4852; eval_time dispatcher :4978-5004, prompt_eval_time :4854-4976); not the path a model runs (that one
- * quantizes the activations, above), kept as a plain form: the weights are read once per activation row. */
+ * quantizes the activations, above), kept as a plain form: the weights are read once per activation row.  One row of a long K
+ * (M == 1, K split over workgroups as in the mat-vec) goes through the library's per-device scratch: two such calls must not overlap
+ * on one GPU. */
 int nh_q8_0_mul_mat_f32_activations(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* stream);
 
 /* One entry of a batch: y[M][N] = mul_mat(W_tiled [N x K], x fp32 [M][K]).  reuse_quantized_x != 0 lets the runner
