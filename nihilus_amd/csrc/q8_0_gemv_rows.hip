@@ -203,6 +203,11 @@ hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, 
 	while (tiles_for(p.splits) > 2 && strips * M * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
 		p.splits *= 2;
 	}
+	// few strips (k/v-sized outputs): keep cutting K while the launch would leave half the CUs without a workgroup and a wave
+	// still owns more than one group
+	while (strips * p.splits < 128 && tiles_for(p.splits) > 1 && strips * M * p.splits * 2 <= GEMV_MAX_SPLIT_UNITS) {
+		p.splits *= 2;
+	}
 	if (p.splits > 1 && stream_is_capturing(s)) { // replay-safe form: no K split, chunked walk instead
 		p.splits = 1;
 	}

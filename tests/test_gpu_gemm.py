@@ -90,7 +90,7 @@ def test_mul_mat_fused(q8, oracle):
         assert rel_l2(got, want) <= REL_L2_TOL
 
 
-@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (14336, 4096), (33, 128), (100, 1024), (8192, 28672), (1024, 8192), (40000, 8192), (64, 128 * 70)])
+@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (14336, 4096), (33, 128), (100, 1024), (8192, 28672), (1024, 8192), (1024, 4096), (512, 2048), (40000, 8192), (64, 128 * 70)])
 def test_mul_mat_few_rows(q8, oracle, n, k):
     # 2 or 3 activation rows: the streaming mat-vec with one dot product per row and weight tile, quantize inside the kernel
     # (unsplit, K split over workgroups, chunked walk, ragged N); no workspace is needed there.  4 and 5 rows: the same kernel on
