@@ -33,5 +33,26 @@ def build_host_tests() -> str:
     return HOST_TEST_BIN
 
 
+FUZZ_SRC = os.path.join(HERE, "fuzz_gguf.cpp")
+FUZZ_BIN = os.path.join(HERE, "fuzz_gguf")
+
+
+def build_gguf_fuzz() -> str:
+    """The GGUF reader's source compiled with AddressSanitizer + UBSan into a mutation driver (host code only; the upload path's
+    HIP and tile symbols resolve against the built library and are never called)."""
+    from nihilus_amd.build import CSRC, PKG_DIR
+
+    cmd = [
+        "g++", "-std=c++20", "-g", "-O1", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-D__HIP_PLATFORM_AMD__",
+        "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", FUZZ_SRC, os.path.join(CSRC, "gguf_q8_0.cpp"), "-o", FUZZ_BIN,
+        "-L", PKG_DIR, "-lnihilus_q8_hip", "-L", "/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/../../nihilus_amd", "-Wl,-rpath,/opt/rocm/lib",
+    ]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"fuzz driver build failed:\n{' '.join(cmd)}\n{res.stderr}")
+    return FUZZ_BIN
+
+
 if __name__ == "__main__":
     print(build_host_tests())
+    print(build_gguf_fuzz())

@@ -153,3 +153,22 @@ def test_rejects_malformed_files(gguf, oracle, tmp_path):
     W.write_gguf(p, [("a", W.U8, 5)], [])
     with gguf.GGUFFile(p) as f:
         assert f.tensor_count == 0
+
+
+def test_mutated_files_under_sanitizers(oracle, tmp_path):
+    # 6000 mutants of a valid file (truncated, flipped bytes and bits, overwritten counts / lengths / offsets) through every query of the
+    # reader, in a build of its source with AddressSanitizer and UBSan: no report, and no accepted tensor may reach past the end of its file
+    import subprocess
+    import sys
+
+    sys.path.insert(0, os.path.join(ROOT, "tests", "cpp"))
+    import build_host_tests as B
+
+    if not os.path.exists(B.FUZZ_BIN) or os.path.getmtime(B.FUZZ_BIN) < max(os.path.getmtime(B.FUZZ_SRC), os.path.getmtime(os.path.join(ROOT, "nihilus_amd", "csrc", "gguf_q8_0.cpp"))):
+        B.build_gguf_fuzz()
+    path, _, _ = model_file(tmp_path, oracle)
+    for seed in (1, 2):
+        res = subprocess.run([B.FUZZ_BIN, path, "3000", str(seed), str(tmp_path / "mutant.gguf")], capture_output=True, text=True, timeout=240)
+        assert res.returncode == 0, (res.stdout + res.stderr)[-3000:]
+        assert "3000 mutants" in res.stdout and "ERROR" not in res.stderr
+        assert int(res.stdout.split(",")[1].split()[0]) > 300  # a fair share of the mutants still parses: the queries really ran
