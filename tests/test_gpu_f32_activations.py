@@ -8,7 +8,7 @@ from helpers import REL_L2_TOL, random_blocks, rel_l2, to_dev, to_host
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (1, 1000, 14336), (1, 33, 128), (3, 257, 1024), (40, 96, 512), (2, 14336, 4096), (1, 64, 0), (2, 160, 5120), (1, 96, 8192), (1, 64, 28672), (1, 40, 4224)])
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (1, 1000, 14336), (1, 33, 128), (3, 257, 1024), (40, 96, 512), (2, 14336, 4096), (1, 64, 0), (2, 160, 5120), (1, 96, 8192), (1, 64, 28672), (1, 40, 4224), (2, 96, 14336), (3, 64, 28672)])
 def test_matches_checker(q8, oracle, m, n, k):
     rng = np.random.default_rng(m + n + k)
     w = random_blocks(rng, n, k) if k else np.zeros(0, dtype=np.uint8)
