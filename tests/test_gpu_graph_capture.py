@@ -33,7 +33,8 @@ def test_captured_launches_replay_with_new_inputs(q8, oracle):
     res = to_dev(rng.standard_normal(n_out).astype(np.float32))
 
     def launches():
-        return (q8.gemv_f32(w, x1, n, k), q8.mul_mat(w, x8[:3], n, k), q8.mul_mat(w, x8, n, k), q8.ffn(wg, wu, wd, xf, n_ff, kf, n_out, residual=res))
+        return (q8.gemv_f32(w, x1, n, k), q8.mul_mat(w, x8[:3], n, k), q8.mul_mat(w, x8, n, k), q8.ffn(wg, wu, wd, xf, n_ff, kf, n_out, residual=res),
+                q8.mul_mat_f32_activations(w, x1, n, k))  # one row of a long K: split over workgroups eagerly, unsplit under capture
 
     def new_inputs(seed):
         x8.copy_(to_dev(oracle.fill_activations(seed, 8 * k).reshape(8, k)))
@@ -57,6 +58,7 @@ def test_captured_launches_replay_with_new_inputs(q8, oracle):
             assert rel_l2(g, e) < 2e-6, (seed, i)  # same arithmetic, different cut of K
         assert rel_l2(got[3], want[3]) <= 1e-3, seed  # a quantizer sits between the FFN's stages
         assert np.isfinite(got[3]).all()
+        assert rel_l2(got[4], want[4]) < 2e-6, seed
     # and against the checker once, so that "equal to eager" cannot hide a common mistake
     aq = oracle.quantize_rows(to_host(x1))[0]
     assert rel_l2(got[0], oracle.gemv(to_host(q8.untile(w, n, k)), aq, n, k)) <= REL_L2_TOL
