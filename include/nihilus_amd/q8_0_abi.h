@@ -143,6 +143,16 @@ int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_
 /* The same with the residual add of the layer behind it (attn_out mul_mat -> residual add, infra/core_traits.hpp:768-772):
  * y = W . Q(x) + residual, one fp32 add after the row's sum.  residual may be y itself (in-place accumulate). */
 int nh_q8_0_gemv_tiled_residual_f32(const void* W_tiled, const float* x, const float* residual, float* y, int64_t N, int64_t K, void* stream);
+/* nh_q8_0_gemv_tiled_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): same kernels, same cut of the matrix, same bits in y, but the partial sums that a K split
+ * hands between workgroups go through a 512 KiB array that is part of the library's code object (one copy per GPU, held until
+ * the process ends) instead of a buffer allocated on first use.  The call allocates and frees nothing.  A shape whose cut
+ * needs more than NH_Q8_0_NOALLOC_MAX_SPLIT_UNITS (32-row strip, K part) slots is rejected with NH_ERR_TOO_LARGE before
+ * anything is launched ([4096 x 14336] uses 512, [8192 x 28672] 2048; shapes that need no K split always fit).  Every call on
+ * a GPU shares that GPU's array: two such calls must not overlap on one GPU (run them on one stream).  No counterpart in the
+ * reference, whose kernels never allocate (infra/model.hpp:241 owns the arena). */
+#define NH_Q8_0_NOALLOC_MAX_SPLIT_UNITS 2048
+int nh_q8_0_gemv_tiled_f32_noalloc(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream);
 /* The same for up to 3 weight matrices that share K and x (q/k/v, gate/up: infra/core_traits.hpp:575-594, :976-986)
  * as ONE launch: y[i] = W_tiled[i] . quantize(x), i < count.  host_* arrays are host memory, read before return. */
 int nh_q8_0_gemv_tiled_multi_f32(const void* const* host_W_tiled, float* const* host_y, const int64_t* host_N, int64_t count, const float* x, int64_t K, void* stream);

@@ -452,6 +452,22 @@ int nh_q8_0_gemv_tiled_f32(const void* W_tiled, const float* x, float* y, int64_
 	return nh_q8_0_gemv_tiled_multi_f32(&W_tiled, &y, &N, 1, x, K, stream);
 }
 
+int nh_q8_0_gemv_tiled_f32_noalloc(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream) {
+	NH_TRY(check_shape(N, 0, K, true));
+	if (N == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(y, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(y), NH_ERR_ALIGNMENT);
+	if (K > 0) {
+		NH_REQUIRE(W_tiled && x, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(W_tiled) && aligned16(x), NH_ERR_ALIGNMENT);
+		NH_REQUIRE(nh::gemv_noalloc_fits(N, K), NH_ERR_TOO_LARGE); // the K split's partial sums would not fit the built-in array
+	}
+	NH_TRY(require_device());
+	return from_hip(nh::launch_gemv_tiled_f32_noalloc(W_tiled, x, y, N, K, as_stream(stream)));
+}
+
 int nh_q8_0_debug_fused_norm_quantize(const float* x, const float* norm_weight, float eps, void* xq_blocks_out, int64_t K, void* stream) {
 	NH_TRY(check_shape(1, 0, K, true));
 	if (K == 0) {

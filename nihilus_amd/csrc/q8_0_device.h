@@ -248,10 +248,14 @@ hipError_t launch_gemv(const void* W, const void* xq_blocks, float* y, int32_t* 
 constexpr int GEMV_MAX_SEGMENTS = 3;
 hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, hipStream_t s,
 	const float* norm_w = nullptr, float norm_eps = 0.0f, const float* const* residual = nullptr);
-// Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
+// The fused quantize + mat-vec of one matrix with the K-split hand-off going through a device array that is part of the
+// code object: nothing is allocated.  gemv_noalloc_fits says whether the shape's cut fits that array.
+bool gemv_noalloc_fits(int64_t N, int64_t K);
+hipError_t launch_gemv_tiled_f32_noalloc(const void* W, const float* x, float* y, int64_t N, int64_t K, hipStream_t s);
 hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* norm_w, float norm_eps, const float* residual, float* y, int64_t n_ff,
 	int64_t K, int64_t n_out, hipStream_t s);
 hipError_t copy_ffn_gate_up(float* gate_out, float* up_out, int64_t n_ff, hipStream_t s);
+// Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w = nullptr, float norm_eps = 0.0f);
 // fp32 activations [M][K] against tiled Q8_0 weights without quantizing the activations (the reference's <float, block_q8_0, float>
 // mul_mat, cpu/avx_2.hpp:4782-5004): y [M][N].  K == 0 gives zeros.

@@ -237,6 +237,72 @@ hipError_t prepare_gemv_scratch() {
 	return get_gemv_scratch(&sc);
 }
 
+// ---- the mat-vec for callers that must not allocate -------------------------------------------------------------
+// Same kernels, same cut, same hand-off; the tagged partial sums of a K split live in a device array that is part of the
+// code object instead of a buffer made with hipMalloc.  Every GPU the library runs on holds its own copy of the array
+// at its own address for the life of the process; its name below is only the host-side handle for hipGetSymbolAddress.
+constexpr int NOALLOC_MAX_SPLIT_UNITS = 2048; // (strip, split) slots: 512 KiB
+static __device__ __align__(256) uint64_t scratch[NOALLOC_MAX_SPLIT_UNITS * STRIP_ROWS];
+
+__global__ void clear_tags_kernel(uint64_t* __restrict__ p, int n) {
+	const int i = static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+	if (i < n) {
+		p[i] = 0ull;
+	}
+}
+
+// The array's device address and the next epoch, per device.  First use on a device (that device current): look the
+// address up, then set every tag to zero, the one value no launch uses as its epoch (a fill kernel, not a memset node).
+// Calls that overlap on one GPU share the array and race on it, like the calls that share the allocated scratch.
+static hipError_t get_noalloc_scratch(gemv_scratch* out, hipStream_t s) {
+	struct state {
+		uint64_t* ptr  = nullptr;
+		unsigned epoch = 0;
+	};
+	static std::mutex lock;
+	static state per_device[64];
+	int dev		 = 0;
+	hipError_t e = hipGetDevice(&dev);
+	if (e != hipSuccess) {
+		return e;
+	}
+	if (dev < 0 || dev >= 64) {
+		return hipErrorInvalidDevice;
+	}
+	std::lock_guard<std::mutex> g(lock);
+	state& st = per_device[dev];
+	if (!st.ptr) {
+		void* p = nullptr;
+		e		= hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+		if (e != hipSuccess) {
+			return e;
+		}
+		if (!p) {
+			return hipErrorInvalidSymbol;
+		}
+		constexpr int n = NOALLOC_MAX_SPLIT_UNITS * STRIP_ROWS;
+		clear_tags_kernel<<<dim3((n + 255) / 256), dim3(256), 0, s>>>(static_cast<uint64_t*>(p), n); // stream order puts it ahead of the launch that follows
+		e = hipGetLastError();
+		if (e != hipSuccess) {
+			return e;
+		}
+		st.ptr = static_cast<uint64_t*>(p);
+	}
+	++st.epoch;
+	if (st.epoch == 0) {
+		++st.epoch;
+	}
+	*out		= gemv_scratch{};
+	out->tagged = st.ptr;
+	out->epoch	= st.epoch;
+	return hipSuccess;
+}
+
+bool gemv_noalloc_fits(int64_t N, int64_t K) {
+	const gemv_plan p = plan_gemv((N + STRIP_ROWS - 1) / STRIP_ROWS, K);
+	return p.splits == 1 || static_cast<int64_t>(p.strips) * p.splits <= NOALLOC_MAX_SPLIT_UNITS;
+}
+
 template<int TILES, bool XF32, bool LOOP, bool NORM, int RS = 1> static hipError_t launch_gemv_tiled_n(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
 	const dim3 grid(static_cast<unsigned>(p.strips * p.splits * RS)), block(GEMV_WAVES * 64);
 	if constexpr (RS > 1) { // row split (unsplit K, production only): RS workgroups per strip, nothing handed over
@@ -280,7 +346,7 @@ template<int RS, bool XF32> static hipError_t launch_gemv_tiled_rs(int tiles, co
 }
 
 static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, const int64_t* N, int count, const void* x, bool x_is_f32, int64_t K, void* dump, int dump_mode, hipStream_t s,
-	const float* norm_w = nullptr, float norm_eps = 0.0f, const float* const* residual = nullptr) {
+	const float* norm_w = nullptr, float norm_eps = 0.0f, const float* const* residual = nullptr, bool noalloc = false) {
 	gemv_segments seg{};
 	int64_t strips = 0;
 	for (int i = 0; i < GEMV_MAX_SEGMENTS; ++i) {
@@ -303,7 +369,10 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 	}
 	gemv_scratch sc;
 	if (p.splits > 1) {
-		const hipError_t e = get_gemv_scratch(&sc, true);
+		if (noalloc && p.strips * p.splits > NOALLOC_MAX_SPLIT_UNITS) {
+			return hipErrorInvalidValue; // the caller checks gemv_noalloc_fits first
+		}
+		const hipError_t e = noalloc ? get_noalloc_scratch(&sc, s) : get_gemv_scratch(&sc, true);
 		if (e != hipSuccess) {
 			return e;
 		}
@@ -398,6 +467,18 @@ hipError_t launch_gemv_tiled_multi(const void* const* W, float* const* y, const 
 		return hipGetLastError();
 	}
 	return launch_gemv_tiled_any(W, y, N, count, x, x_is_f32, K, nullptr, DUMP_NONE, s, x_is_f32 ? norm_w : nullptr, norm_eps, residual);
+}
+
+hipError_t launch_gemv_tiled_f32_noalloc(const void* W, const float* x, float* y, int64_t N, int64_t K, hipStream_t s) {
+	if (K == 0) {
+		if (N > 0) {
+			zero_f32_kernel<<<dim3(static_cast<unsigned>((N + 255) / 256)), dim3(256), 0, s>>>(y, N); // empty dot product
+		}
+		return hipGetLastError();
+	}
+	const void* wl[1] = { W };
+	float* yl[1]	  = { y };
+	return launch_gemv_tiled_any(wl, yl, &N, 1, x, true, K, nullptr, DUMP_NONE, s, nullptr, 0.0f, nullptr, true);
 }
 
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w, float norm_eps) {
