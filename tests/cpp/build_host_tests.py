@@ -13,9 +13,11 @@ if ROOT not in sys.path:
 
 HOST_TEST_SRC = os.path.join(HERE, "test_mul_mat_dispatch.cpp")
 HOST_TEST_BIN = os.path.join(HERE, "test_mul_mat_dispatch")
+MEGA_TEST_BIN = os.path.join(HERE, "test_mega_dispatch")  # the live dispatch point (core_types key), run on the GPU
+REFERENCE_MODE_BIN = os.path.join(HERE, "test_reference_mode_compiles")  # the headers against the reference's own primary template
 
 
-def build_host_tests() -> str:
+def _build_one(src: str, out: str) -> str:
     from nihilus_amd.build import PKG_DIR, hipcc
 
     cxx = os.path.join(os.path.dirname(hipcc()), "amdclang++")
@@ -23,14 +25,20 @@ def build_host_tests() -> str:
         cxx = "/opt/rocm/bin/amdclang++"
     oracle_dir = os.path.join(ROOT, "oracle")
     cmd = [
-        cxx, "-std=c++23", "-O2", "-Wall", "-Wextra", "-I", os.path.join(ROOT, "include"), HOST_TEST_SRC, "-o", HOST_TEST_BIN,
+        cxx, "-std=c++23", "-O2", "-Wall", "-Wextra", "-I", os.path.join(ROOT, "include"), os.path.join(HERE, src), "-o", out,
         "-L", PKG_DIR, "-lnihilus_q8_hip", "-L", oracle_dir, "-lq8_0_oracle",
         "-Wl,-rpath,$ORIGIN/../../nihilus_amd", "-Wl,-rpath,$ORIGIN/../../oracle", "-Wl,-rpath,/opt/rocm/lib",
     ]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"host test build failed:\n{' '.join(cmd)}\n{res.stderr}")
-    return HOST_TEST_BIN
+    return out
+
+
+def build_host_tests() -> str:
+    _build_one("test_mega_dispatch.cpp", MEGA_TEST_BIN)
+    _build_one("test_reference_mode_compiles.cpp", REFERENCE_MODE_BIN)
+    return _build_one("test_mul_mat_dispatch.cpp", HOST_TEST_BIN)
 
 
 FUZZ_SRC = os.path.join(HERE, "fuzz_gguf.cpp")

@@ -26,6 +26,9 @@ struct test_config {
 	static constexpr bool exceptions{ true };
 	static constexpr bool synchronous{ true }; // sync after each launch, as the reference's GPU path does
 	static constexpr uint64_t max_sequence_length{ 64 };
+	struct model_traits_type {
+		static constexpr uint32_t block_count{ 32 };
+	};
 };
 
 // LLaMA-3-8B k-projection shape (infra/model_traits.hpp:49-65, infra/core_traits.hpp:583-584): W [K = 4096, N = 1024]
@@ -34,17 +37,17 @@ using weight_type	  = core_trait_dims<K, N, 1, 1>;
 using activation_type = core_trait_dims<K, test_config::max_sequence_length, 1, 1, 1>; // dim1 = sequence length, runtime
 using output_dims	  = core_trait_dims<N, test_config::max_sequence_length, 1, 1, 1>;
 
-struct k_mul_mat_op : kernel_traits_old<test_config, output_dims, kernel_types::mul_mat, float, weight_type, activation_type>, data_mixin<data_strategy_types::global, 32> {};
+struct k_mul_mat_op : kernel_traits_old<test_config, output_dims, kernel_types::mul_mat, float, weight_type, activation_type>, data_mixin<test_config, data_strategy_types::global, float> {};
 
 static_assert(k_mul_mat_op::input_01_dims[0] == K && k_mul_mat_op::output_dims[0] == N);
-static_assert(arch_index<device_types::gpu> == 5);
+static_assert(arch_index<device_types::gpu> == 5 && gfx950_arch_index == 5);
 static_assert(runtime_dims_t<k_mul_mat_op>);
 static_assert(sizeof(block_q8_0<half>) == NH_Q8_0_BLOCK_BYTES && Q_SIZE == NH_Q8_0_QK);
 
 // token embeddings: table [K, N rows] (the k-projection bytes stand in for an embedding table), ids [tokens], out [K, tokens]
 using ids_type		= core_trait_dims<test_config::max_sequence_length, 1, 1, 1>;
 using embd_out_dims = core_trait_dims<K, test_config::max_sequence_length, 1, 1, 1>;
-struct get_rows_op : kernel_traits_old<test_config, embd_out_dims, kernel_types::get_rows, float, weight_type, ids_type>, data_mixin<data_strategy_types::global, 32> {};
+struct get_rows_op : kernel_traits_old<test_config, embd_out_dims, kernel_types::get_rows, float, weight_type, ids_type>, data_mixin<test_config, data_strategy_types::global, float> {};
 using embd_eval_dispatch   = get_rows_dispatcher<test_config, processing_phases::eval_time, get_rows_op>;
 using embd_prompt_dispatch = get_rows_dispatcher<test_config, processing_phases::prompt_eval_time, get_rows_op>;
 
@@ -150,8 +153,8 @@ int main(int argc, char** argv) {
 
 	// the key the reference implements on the CPU, <float, block_q8_0<half>, float>: fp32 activations, no activation quantize
 	{
-		using f32_eval	 = kernel_dispatcher_impl<test_config, k_mul_mat_op, device_types::gpu, 5, kernel_types::mul_mat, processing_phases::eval_time, k_mul_mat_op, float, block_q8_0<half>, float>;
-		using f32_prompt = kernel_dispatcher_impl<test_config, k_mul_mat_op, device_types::gpu, 5, kernel_types::mul_mat, processing_phases::prompt_eval_time, k_mul_mat_op, float, block_q8_0<half>,
+		using f32_eval	 = per_op_kernel_dispatcher_impl<test_config, k_mul_mat_op, device_types::gpu, 5, kernel_types::mul_mat, processing_phases::eval_time, k_mul_mat_op, float, block_q8_0<half>, float>;
+		using f32_prompt = per_op_kernel_dispatcher_impl<test_config, k_mul_mat_op, device_types::gpu, 5, kernel_types::mul_mat, processing_phases::prompt_eval_time, k_mul_mat_op, float, block_q8_0<half>,
 			float>;
 		std::vector<float> want_f(M * N), got_f(M * N);
 		nho_mul_mat_q8_f32(w.data(), x.data(), want_f.data(), 1, N, K, 0); // the eval_time leaf's order

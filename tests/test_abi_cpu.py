@@ -139,6 +139,33 @@ def test_cpp_dispatch_surface_compiles_and_static_checks_hold():
     assert res.returncode == 0 and "static checks ok" in res.stdout
 
 
+def test_cpp_live_dispatch_point_compiles_against_the_reference_declaration():
+    # mega_dispatch.hpp / mul_mat_dispatch.hpp with NIHILUS_AMD_WITH_REFERENCE_HEADERS: every reference name comes from a
+    # test-local header whose primary template is the reference's own declaration of the live specialisation point; all eight
+    # specialisations are instantiated through the reference's caller-side template.  Also the stand-alone build's static checks.
+    b = _host_tests()
+    if not (os.path.exists(b.REFERENCE_MODE_BIN) and os.path.exists(b.MEGA_TEST_BIN)):
+        import oracle  # noqa: F401
+
+        b.build_host_tests()
+    res = subprocess.run([b.REFERENCE_MODE_BIN], capture_output=True, text=True)
+    assert res.returncode == 0 and "reference-mode build ok" in res.stdout
+    res = subprocess.run([b.MEGA_TEST_BIN, "--compile-only-check"], capture_output=True, text=True)
+    assert res.returncode == 0 and "static checks ok" in res.stdout
+    # the mode switch is real: the headers must not pull the mirror in when the reference's names are already there
+    text = open(os.path.join(ROOT, "include", "nihilus_amd", "mul_mat_dispatch.hpp")).read()
+    assert re.search(r"#ifndef NIHILUS_AMD_WITH_REFERENCE_HEADERS\s+#include \"reference_mirror.hpp\"", text)
+
+
+@pytest.mark.gpu
+def test_cpp_live_dispatch_point_on_gpu():
+    # the four mega cores, both phases, through kernel_dispatcher<config, phase, core>::impl on a two-block graph
+    b = _host_tests()
+    res = subprocess.run([b.MEGA_TEST_BIN], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert "mega dispatch ok" in res.stdout
+
+
 @pytest.mark.gpu
 def test_cpp_dispatch_surface_on_gpu():
     b = _host_tests()
