@@ -14,6 +14,17 @@
  * called from infra/monolithic_dispatcher.hpp:41-63).  The C++ header mul_mat_dispatch.hpp supplies
  * those specialisations for device_types::gpu and forwards to the functions below.
  *
+ * Streams
+ *   Launches that hand data between workgroups do so through scratch memory that the library keeps per GPU (made on first
+ *   use or by nh_q8_0_prepare): nh_q8_0_gemv_tiled*, nh_q8_0_gemv_tiled_group_f32, nh_q8_0_mul_mat*, nh_q8_0_mul_mat_batch,
+ *   nh_q8_0_mul_mat_f32_activations (each when the shape makes them split K over workgroups), nh_q8_0_gemm_tiled* for M <= 64,
+ *   and nh_q8_0_ffn_f32 always.  That scratch serves ONE stream at a time per GPU: enqueue such calls on one stream, or let
+ *   the other stream drain first.  A call that would use the scratch while a launch from a different stream may still be
+ *   running returns NH_ERR_BUSY and launches nothing (not detected: work on a capturing stream, work that followed a
+ *   launch on the NULL stream, and replays of captured graphs, which the caller must keep from overlapping).
+ *   A kernel that waits for another workgroup's data does so for a bounded time; if it gives up, the output holds NaN and
+ *   the next nh_stream_sync (or nh_q8_0_last_error) on that GPU returns NH_ERR_DEVICE_TIMEOUT once.
+ *
  * Data layouts
  *   "blocks"  the reference's wire layout: rows of packed 34-byte block_q8_0 { fp16 d; int8 qs[32] }
  *             (common/data_types.hpp:38-44), row stride (K/32)*34 bytes, row-major.
@@ -48,7 +59,9 @@ typedef enum nh_status {
 	NH_ERR_ARGUMENT	   = -6, /* any other invalid argument */
 	NH_ERR_IO		   = -7, /* a file could not be opened or mapped */
 	NH_ERR_FORMAT	   = -8, /* a file is not what its reader accepts */
-	NH_ERR_NOT_FOUND   = -9 /* no tensor or metadata key of that name */
+	NH_ERR_NOT_FOUND   = -9, /* no tensor or metadata key of that name */
+	NH_ERR_BUSY		   = -10, /* the per-device scratch is still in use by a launch on ANOTHER stream: nothing was launched (see "Streams" below) */
+	NH_ERR_DEVICE_TIMEOUT = -11 /* reported by nh_stream_sync / nh_q8_0_last_error: a kernel gave up a bounded wait, its output holds NaN */
 } nh_status;
 
 /* Library / device ------------------------------------------------------------------------------ */
@@ -67,9 +80,15 @@ int nh_malloc(void** host_out_dev_ptr, int64_t bytes);
 int nh_free(void* dev_ptr);
 int nh_memcpy_h2d(void* dst_dev, const void* host_src, int64_t bytes, void* stream);
 int nh_memcpy_d2h(void* host_dst, const void* src_dev, int64_t bytes, void* stream);
+/* hipMemsetAsync: not for a stream that is being captured into a HIP graph (it would record a memset node; every launch entry
+ * point of this library clears memory with fill kernels instead and can be captured). */
 int nh_memset(void* dst_dev, int value, int64_t bytes, void* stream);
-/* Blocks until the stream has drained: the cudaDeviceSynchronize after each launch in cuda/cuda_12.hpp:679. */
+/* Blocks until the stream has drained: the cudaDeviceSynchronize after each launch in cuda/cuda_12.hpp:679.  Returns
+ * NH_ERR_DEVICE_TIMEOUT (once) if a kernel on this GPU gave up a bounded wait since the last report. */
 int nh_stream_sync(void* stream);
+/* Reads and clears the GPU's sticky device-side error without waiting for anything: NH_OK or NH_ERR_DEVICE_TIMEOUT.  The
+ * reference looks at the device's error state after a launch only in dev builds (cuda/cuda_12.hpp:650-655). */
+int nh_q8_0_last_error(void);
 /* Allocates, for the current device, the two internal scratch buffers that K-split launches hand partial sums through
  * (about 2.6 MiB and 16 MiB; otherwise made by the first launch that needs one).  After it no launch entry point of this library
  * allocates device memory: call it once per device before capturing launches into a HIP graph or entering a serving loop.
@@ -271,6 +290,11 @@ int nh_q8_0_debug_fused_norm_quantize(const float* x, const float* norm_weight, 
 /* The gate and up projections' fp32 outputs of the last nh_q8_0_ffn_f32 on this device (they never leave the
  * library otherwise), copied out for comparison. */
 int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void* stream);
+
+/* How many polls a workgroup of nh_q8_0_ffn_f32 waits for another workgroup's data before it gives up (default and upper
+ * limit 2^20, lower limit 1).  Test hook for the time-out report: with a limit of 1 the down projection's workgroups find
+ * their activation missing and give up while every kernel still runs to its end.  Process-wide. */
+int nh_q8_0_debug_set_spin_limit(int64_t polls);
 
 /* Synthetic inputs (benchmark / test utility) --------------------------------------------------- */
 

@@ -327,7 +327,11 @@ int nh_gguf_open(const char* path, nh_gguf** out) {
 	for (size_t i = 0; i < f->tensors.size(); ++i) {
 		nh_gguf_tensor_info& t = f->tensors[i];
 		t.name				   = f->names[i].c_str();
-		t.file_offset		   = f->data_start + t.offset;
+		// checked before the addition: an offset close to 2^64 would wrap to a small file offset that passes the range checks below
+		if (t.offset > f->size - f->data_start) {
+			return fail(NH_ERR_FORMAT);
+		}
+		t.file_offset = f->data_start + t.offset;
 		if (t.offset % f->alignment != 0 || t.file_offset > f->size || t.byte_size > f->size - t.file_offset) {
 			return fail(NH_ERR_FORMAT);
 		}
@@ -507,6 +511,11 @@ int nh_gguf_upload_tensor(const nh_gguf* f, const nh_gguf_tensor_info* info, voi
 	const void* src = nh_gguf_tensor_data(f, info);
 	if (!src || info->byte_size == 0) {
 		return NH_ERR_ARGUMENT; // not a tensor of this file, or a type without a known size
+	}
+	// the caller owns this copy of the record and may have edited it: the byte count must still be the one its type and dims give,
+	// or the tile kernel would read past the staging slice
+	if (info->n_dims == 0 || info->n_dims > 4 || nh_ggml_tensor_bytes(info->ggml_type, info->dims, info->n_dims) != static_cast<int64_t>(info->byte_size)) {
+		return NH_ERR_ARGUMENT;
 	}
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	if (!tiled) {

@@ -2,7 +2,7 @@
 // Nothing here computes; every rejected argument returns a negative nh_status before any launch, so a
 // malformed call can never reach a kernel with shapes the kernel does not expect.
 #include "../../include/nihilus_amd/q8_0_abi.h"
-#include "q8_0_device.h"
+#include "q8_0_gemv_tiled.h"
 
 #include <cstring>
 
@@ -20,6 +20,9 @@ inline hipStream_t as_stream(void* s) {
 	return static_cast<hipStream_t>(s);
 }
 inline int from_hip(hipError_t e) {
+	if (e == hipErrorNotReady) {
+		return NH_ERR_BUSY; // the only source: the per-device scratch is still in use by a launch on another stream
+	}
 	return e == hipSuccess ? NH_OK : static_cast<int>(e);
 }
 
@@ -103,6 +106,10 @@ const char* nh_status_string(int status) {
 			return "file format not accepted";
 		case NH_ERR_NOT_FOUND:
 			return "name not found";
+		case NH_ERR_BUSY:
+			return "the library's per-device scratch is still in use by a launch on another stream";
+		case NH_ERR_DEVICE_TIMEOUT:
+			return "a kernel gave up a bounded wait for data from another workgroup (its output holds NaN)";
 		default:
 			return status > 0 ? hipGetErrorString(static_cast<hipError_t>(status)) : "unknown status";
 	}
@@ -181,7 +188,19 @@ int nh_memset(void* dst_dev, int value, int64_t bytes, void* stream) {
 
 int nh_stream_sync(void* stream) {
 	NH_TRY(require_device());
-	return from_hip(hipStreamSynchronize(as_stream(stream)));
+	NH_TRY(from_hip(hipStreamSynchronize(as_stream(stream))));
+	return nh::take_device_error() != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
+}
+
+int nh_q8_0_last_error(void) {
+	NH_TRY(require_device());
+	return nh::take_device_error() != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
+}
+
+int nh_q8_0_debug_set_spin_limit(int64_t polls) {
+	NH_REQUIRE(polls >= 1, NH_ERR_ARGUMENT);
+	nh::set_published_spin_limit(polls > nh::PUBLISHED_SPIN_LIMIT ? nh::PUBLISHED_SPIN_LIMIT : static_cast<int>(polls));
+	return NH_OK;
 }
 
 int64_t nh_q8_0_blocks_bytes(int64_t rows, int64_t K) {
@@ -508,7 +527,9 @@ static int gemm_common(const void* W, const void* A, float* C, int64_t M, int64_
 	if (M == 0 || N == 0) {
 		return NH_OK;
 	}
-	NH_REQUIRE(M <= 65535 * 128, NH_ERR_TOO_LARGE); // grid.y
+	// grid.y of the kernel that will run: the MFMA tile kernel covers 64 rows per workgroup row (two 32-row strips), the streaming
+	// kernel 32 or 64, the kernel on packed blocks 128
+	NH_REQUIRE(M <= 65535 * (tiled ? 32 : 128), NH_ERR_TOO_LARGE);
 	NH_REQUIRE(C, NH_ERR_NULL_POINTER);
 	NH_REQUIRE(aligned16(C) && aligned16(residual), NH_ERR_ALIGNMENT);
 	if (K > 0) {

@@ -43,6 +43,8 @@ struct ffn_args {
 	int producers; // n_ff / 32
 	int p_per_slot, p_rem; // a producer strip's K range over the 8 waves of one matrix
 	int split_shift; // a consumer strip's K range goes over (1 << split_shift) workgroups of 16 waves
+	unsigned* error_word; // device-visible host word: set when a consumer gives up waiting for a producer
+	int spin_limit; // polls before it does
 };
 
 template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
@@ -124,10 +126,10 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 	const int row_l		   = gstrip * STRIP_ROWS + (lane & 31);
 	float acc			   = 0.0f;
 	if constexpr (!LOOP) {
-		acc = gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_words, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_c, lane, row_l, a.n_out, false, a.epoch);
+		acc = gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_words, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_c, lane, row_l, a.n_out, false, a.epoch, nullptr, 0, a.spin_limit);
 	} else {
 		for (int gc = g0; gc < g1; gc += TILES) {
-			acc += gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_words, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_c, lane, row_l, a.n_out, false, a.epoch);
+			acc += gemv_chunk<TILES, X_PUBLISHED, DUMP_NONE>(w_strip, a.act_words, a.error_word, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_c, lane, row_l, a.n_out, false, a.epoch, nullptr, 0, a.spin_limit);
 			__builtin_amdgcn_wave_barrier();
 		}
 	}
@@ -180,7 +182,7 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 		return hipGetLastError();
 	}
 	gemv_scratch sc;
-	const hipError_t e = get_gemv_scratch(&sc, true);
+	const hipError_t e = get_gemv_scratch(&sc, true, s);
 	if (e != hipSuccess) {
 		return e;
 	}
@@ -226,6 +228,8 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	a.act_words	 = sc.act_words;
 	a.epoch		 = sc.epoch;
 	a.tagged	 = sc.tagged;
+	a.error_word = sc.error_word;
+	a.spin_limit = sc.spin_limit;
 	a.n_ff		 = static_cast<int>(n_ff);
 	a.n_out		 = static_cast<int>(n_out);
 	a.groups_p	 = static_cast<int>(K / GROUP_K);

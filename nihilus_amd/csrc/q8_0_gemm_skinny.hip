@@ -257,8 +257,13 @@ constexpr int SK_MAX_SPLIT_STRIPS = 512;
 struct skinny_scratch {
 	float* partials	   = nullptr;
 	unsigned* counters = nullptr;
+	hipStream_t user   = nullptr; // stream of the last K-split launch
+	bool has_user	   = false;
 };
-static hipError_t get_skinny_scratch(skinny_scratch* out) {
+// launching = true: a K-split launch on `s` is about to use the scratch.  It serves one stream at a time: if the previous such
+// launch went to another stream that has not drained, hipErrorNotReady comes back (NH_ERR_BUSY at the C ABI).  Not checked for
+// capturing streams or after a launch on the null stream (neither may be queried safely).
+static hipError_t get_skinny_scratch(skinny_scratch* out, bool launching = false, hipStream_t s = nullptr) {
 	static std::mutex lock;
 	static skinny_scratch per_device[64];
 	int dev		 = 0;
@@ -287,6 +292,19 @@ static hipError_t get_skinny_scratch(skinny_scratch* out) {
 		sc.partials = static_cast<float*>(p);
 		sc.counters = reinterpret_cast<unsigned*>(static_cast<uint8_t*>(p) + tiles);
 	}
+	if (launching && !stream_is_capturing(s)) {
+		if (sc.has_user && sc.user != s && sc.user != nullptr && !stream_is_capturing(sc.user)) {
+			const hipError_t q = hipStreamQuery(sc.user);
+			if (q == hipErrorNotReady) {
+				return q;
+			}
+			if (q != hipSuccess) {
+				(void)hipGetLastError();
+			}
+		}
+		sc.user		= s;
+		sc.has_user = true;
+	}
 	*out = sc;
 	return hipSuccess;
 }
@@ -313,7 +331,7 @@ template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8
 	}
 	skinny_scratch sc;
 	if (splits > 1) {
-		const hipError_t e = get_skinny_scratch(&sc);
+		const hipError_t e = get_skinny_scratch(&sc, true, s);
 		if (e != hipSuccess) {
 			return e;
 		}

@@ -192,9 +192,33 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	}
 }
 
-hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
-	static std::mutex lock;
-	static gemv_scratch per_device[64];
+namespace {
+	struct scratch_state {
+		gemv_scratch sc;
+		hipStream_t user = nullptr; // stream of the last launch that used the scratch
+		bool has_user	 = false;
+	};
+	std::mutex scratch_lock;
+	scratch_state scratch_per_device[64];
+	int published_spin_limit = PUBLISHED_SPIN_LIMIT;
+
+	// hipErrorNotReady when `prev` still has work in flight; anything else (a destroyed stream, a capturing one) counts as drained
+	hipError_t stream_drained(hipStream_t prev) {
+		if (stream_is_capturing(prev)) {
+			return hipSuccess; // must not be queried; its launches take forms that keep no state in the scratch
+		}
+		const hipError_t q = hipStreamQuery(prev);
+		if (q == hipErrorNotReady) {
+			return q;
+		}
+		if (q != hipSuccess) {
+			(void)hipGetLastError();
+		}
+		return hipSuccess;
+	}
+} // namespace
+
+hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch, hipStream_t s) {
 	int dev		 = 0;
 	hipError_t e = hipGetDevice(&dev);
 	if (e != hipSuccess) {
@@ -203,8 +227,9 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 	if (dev < 0 || dev >= 64) {
 		return hipErrorInvalidDevice;
 	}
-	std::lock_guard<std::mutex> g(lock);
-	gemv_scratch& sc = per_device[dev];
+	std::lock_guard<std::mutex> g(scratch_lock);
+	scratch_state& st = scratch_per_device[dev];
+	gemv_scratch& sc  = st.sc;
 	if (!sc.tagged) {
 		void* p			   = nullptr;
 		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS * 8 + (FFN_MAX_HIDDEN / QK) * BLOCK_BYTES;
@@ -213,23 +238,59 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch) {
 			return e;
 		}
 		e = hipMemset(p, 0, bytes); // synchronous, once: every tag and flag starts at epoch 0, which no launch uses
+		void* word = nullptr;
+		if (e == hipSuccess) {
+			e = hipHostMalloc(&word, 64, hipHostMallocDefault); // pinned, device-visible under the same address
+		}
 		if (e != hipSuccess) {
 			(void)hipFree(p);
 			return e;
 		}
-		sc.tagged  = static_cast<uint64_t*>(p);
-		sc.gate_up = reinterpret_cast<float*>(sc.tagged + static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS);
+		*static_cast<volatile unsigned*>(word) = DEVICE_ERROR_NONE;
+		sc.tagged	  = static_cast<uint64_t*>(p);
+		sc.gate_up	  = reinterpret_cast<float*>(sc.tagged + static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS);
 		sc.act_words  = reinterpret_cast<uint64_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
 		sc.act_blocks = reinterpret_cast<uint8_t*>(sc.act_words + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS); // 16-byte aligned: every part before it is a multiple of 16 bytes
+		sc.error_word = static_cast<unsigned*>(word);
 	}
 	if (next_epoch) {
+		if (!stream_is_capturing(s)) {
+			if (st.has_user && st.user != s && st.user != nullptr) {
+				e = stream_drained(st.user);
+				if (e != hipSuccess) {
+					return e; // hipErrorNotReady: another stream's launch may still be using the scratch
+				}
+			}
+			st.user		= s;
+			st.has_user = true;
+		}
 		++sc.epoch; // tags start at zero and the first epoch handed out is 1
 		if (sc.epoch == 0) {
 			++sc.epoch;
 		}
 	}
-	*out = sc;
+	sc.spin_limit = published_spin_limit;
+	*out		  = sc;
 	return hipSuccess;
+}
+
+unsigned take_device_error() {
+	int dev = 0;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+		(void)hipGetLastError();
+		return DEVICE_ERROR_NONE;
+	}
+	std::lock_guard<std::mutex> g(scratch_lock);
+	unsigned* word = scratch_per_device[dev].sc.error_word;
+	if (!word) {
+		return DEVICE_ERROR_NONE;
+	}
+	return __atomic_exchange_n(word, static_cast<unsigned>(DEVICE_ERROR_NONE), __ATOMIC_RELAXED);
+}
+
+void set_published_spin_limit(int limit) {
+	std::lock_guard<std::mutex> g(scratch_lock);
+	published_spin_limit = limit < 1 ? 1 : (limit > PUBLISHED_SPIN_LIMIT ? PUBLISHED_SPIN_LIMIT : limit);
 }
 
 hipError_t prepare_gemv_scratch() {
@@ -372,7 +433,7 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 		if (noalloc && p.strips * p.splits > NOALLOC_MAX_SPLIT_UNITS) {
 			return hipErrorInvalidValue; // the caller checks gemv_noalloc_fits first
 		}
-		const hipError_t e = noalloc ? get_noalloc_scratch(&sc, s) : get_gemv_scratch(&sc, true);
+		const hipError_t e = noalloc ? get_noalloc_scratch(&sc, s) : get_gemv_scratch(&sc, true, s);
 		if (e != hipSuccess) {
 			return e;
 		}

@@ -146,7 +146,7 @@ hipError_t launch_gemv_group(const gemv_group_op* ops, int count, hipStream_t s)
 	}
 	gemv_scratch sc;
 	if (units > 0) {
-		const hipError_t e = get_gemv_scratch(&sc, true);
+		const hipError_t e = get_gemv_scratch(&sc, true, s);
 		if (e != hipSuccess) {
 			return e;
 		}

@@ -214,7 +214,7 @@ hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, 
 	p.tiles = tiles_for(p.splits);
 	gemv_scratch sc;
 	if (p.splits > 1) {
-		const hipError_t e = get_gemv_scratch(&sc, true);
+		const hipError_t e = get_gemv_scratch(&sc, true, s);
 		if (e != hipSuccess) {
 			return e;
 		}

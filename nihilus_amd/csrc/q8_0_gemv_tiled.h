@@ -27,11 +27,14 @@ enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
 //               whole or not at all, so the data carries its own "ready" mark: the producer needs no acknowledgement
 //               and no flag, the consumer no second read.  The wave first puts all its weight loads in flight, then
 //               reads the 4 * cnt blocks of its slice with device-scope loads until every word carries `epoch`.  The
-//               wait is bounded: after PUBLISHED_SPIN_LIMIT polls the wave gives up and returns NaN, so the kernel
-//               always drains.
+//               wait is bounded: after `spin_limit` polls the wave gives up, returns NaN and stores a non-zero code
+//               in the device-visible error word that `dump` names in this mode (host memory that the next
+//               nh_stream_sync / nh_q8_0_last_error reads), so the kernel always drains and the failure reaches the host.
 enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2 };
 constexpr int PUBLISHED_SPIN_LIMIT = 1 << 20;
 constexpr int PUBLISHED_WORDS	   = 9; // per block: quant dwords 0..7, then the scale
+// codes a kernel leaves in the device-visible error word (nh_q8_0_last_error reports them as NH_ERR_DEVICE_TIMEOUT)
+enum device_error : unsigned { DEVICE_ERROR_NONE = 0, DEVICE_ERROR_PUBLISH_TIMEOUT = 1 };
 
 // RMS norm * weight in front of the quantizer (X_F32 only).  The row's scale needs every element, so the workgroup works it
 // out first, from the row itself (16 KB at K = 4096, served by cache for all but the first workgroups; fixed order of the sum of
@@ -69,7 +72,7 @@ __device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, co
 // hand over between workgroups.
 template<int TILES, int XMODE, int DUMP, bool NORM, int CNT, int RS = 1>
 __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int groups,
-	int lane, int row, int N, bool dump_this_strip, unsigned epoch, gemv_norm* norm, int rowpart = 0) {
+	int lane, int row, int N, bool dump_this_strip, unsigned epoch, gemv_norm* norm, int rowpart = 0, int spin_limit = PUBLISHED_SPIN_LIMIT) {
 	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
 	static_assert(RS == 1 || RS == 2 || RS == 4, "a strip splits into 1, 2 or 4 row parts");
@@ -157,7 +160,7 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 			if (__builtin_amdgcn_ballot_w64(!fresh) == 0) {
 				break;
 			}
-			if (++spins >= PUBLISHED_SPIN_LIMIT) {
+			if (++spins >= spin_limit) {
 				timed_out = true;
 				break;
 			}
@@ -282,7 +285,10 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	}
 	if constexpr (XMODE == X_PUBLISHED) {
 		if (timed_out) {
-			acc = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output
+			acc = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output ...
+			if (lane == 0 && dump) { // ... and to the host (an ordinary vector store to pinned host memory)
+				__hip_atomic_store(static_cast<unsigned*>(dump), static_cast<unsigned>(DEVICE_ERROR_PUBLISH_TIMEOUT), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+			}
 		}
 	}
 	return acc;
@@ -290,11 +296,11 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 
 template<int TILES, int XMODE, int DUMP, bool NORM = false, int RS = 1>
 __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
-	int groups, int lane, int row, int N, bool dump_this_strip, unsigned epoch = 0, gemv_norm* norm = nullptr, int rowpart = 0) {
+	int groups, int lane, int row, int N, bool dump_this_strip, unsigned epoch = 0, gemv_norm* norm = nullptr, int rowpart = 0, int spin_limit = PUBLISHED_SPIN_LIMIT) {
 #define NH_CHUNK_CASE(C)                                                                                                                                              \
 	case C:                                                                                                                                                           \
 		if constexpr (C <= TILES) {                                                                                                                                   \
-			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0), RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart); \
+			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0), RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart, spin_limit); \
 		}                                                                                                                                                             \
 		break;
 	switch (cnt) { // wave-uniform
@@ -306,7 +312,7 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 			break;
 	}
 #undef NH_CHUNK_CASE
-	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0, RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart); // an idle wave (still takes part in barriers)
+	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0, RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart, spin_limit); // an idle wave (still takes part in barriers)
 }
 
 // K split over several workgroups: each publishes the 32 partial sums of its share, tagged with the launch's epoch
@@ -365,8 +371,18 @@ struct gemv_scratch {
 	uint64_t* act_words = nullptr; // [FFN_MAX_HIDDEN / 32][PUBLISHED_WORDS] {epoch, payload}: the quantized activation of the down projection
 	uint8_t* act_blocks = nullptr; // [FFN_MAX_HIDDEN / 32] packed 34-byte blocks: the activation of the three-launch form used under graph capture
 	unsigned epoch	   = 0; // with next_epoch = true: a value no earlier launch on this device has used
+	unsigned* error_word = nullptr; // 4 bytes of pinned host memory the device can write: non-zero once a kernel has given up a bounded wait
+	int spin_limit	   = PUBLISHED_SPIN_LIMIT; // polls before a consumer of published blocks gives up (lowered only by tests)
 };
-hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch = false);
+// next_epoch = true is what a launch that hands data between workgroups through the scratch asks for; `s` is the stream it is
+// about to launch on.  The scratch serves one stream at a time: if the previous such launch went to a different stream and that
+// stream has not drained, hipErrorNotReady comes back (NH_ERR_BUSY at the C ABI) instead of a launch that would corrupt both.
+// The check is skipped for capturing streams and when the previous user was the null stream (which may not be queried while
+// another stream captures).
+hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch = false, hipStream_t s = nullptr);
+// Reads and clears the current device's error word (DEVICE_ERROR_NONE if no scratch exists yet).
+unsigned take_device_error();
+void set_published_spin_limit(int limit);
 
 // How a tiled mat-vec launch is cut: `splits` workgroups per strip, each of 16 waves owning <= `tiles` groups.
 struct gemv_plan {

@@ -120,7 +120,7 @@ hipError_t launch_mul_mat_f32act(const void* W_tiled, const float* x, float* y, 
 			while ((1 << shift) < p.splits) {
 				++shift;
 			}
-			const hipError_t e = get_gemv_scratch(&sc, true);
+			const hipError_t e = get_gemv_scratch(&sc, true, s);
 			if (e != hipSuccess) {
 				return e;
 			}

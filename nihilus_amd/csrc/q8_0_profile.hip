@@ -9,6 +9,7 @@
 #include "../../include/nihilus_amd/q8_0_abi.h"
 #include "q8_0_device.h"
 
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -17,7 +18,7 @@ namespace nh {
 namespace {
 	struct timer_state {
 		std::mutex lock;
-		int kind = -1; // kind being timed, -1 = off
+		std::atomic<int> kind{ -1 }; // kind being timed, -1 = off; read without the lock on every launch
 		std::vector<hipEvent_t> events; // 2 per launch
 		size_t used = 0; // events handed out
 	};
@@ -29,11 +30,11 @@ namespace {
 
 bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop) {
 	timer_state& t = timer();
-	if (t.kind != kind) { // unsynchronised fast path: timing is switched only while no launch is in flight
+	if (t.kind.load(std::memory_order_relaxed) != kind) { // fast path: one relaxed load per launch
 		return false;
 	}
 	std::lock_guard<std::mutex> g(t.lock);
-	if (t.kind != kind || t.used + 2 > t.events.size()) {
+	if (t.kind.load(std::memory_order_relaxed) != kind || t.used + 2 > t.events.size()) {
 		return false;
 	}
 	*start = t.events[t.used];
@@ -52,7 +53,7 @@ int nh_profile_begin(int kernel_kind, int64_t max_launches) {
 	}
 	nh::timer_state& t = nh::timer();
 	std::lock_guard<std::mutex> g(t.lock);
-	if (t.kind != -1) {
+	if (t.kind.load(std::memory_order_relaxed) != -1) {
 		return NH_ERR_ARGUMENT; // already timing
 	}
 	t.events.resize(static_cast<size_t>(max_launches) * 2);
@@ -74,7 +75,7 @@ int nh_profile_begin(int kernel_kind, int64_t max_launches) {
 int nh_profile_end(double* host_total_ms, int64_t* host_launches, double* host_min_ms, double* host_max_ms) {
 	nh::timer_state& t = nh::timer();
 	std::lock_guard<std::mutex> g(t.lock);
-	if (t.kind == -1) {
+	if (t.kind.load(std::memory_order_relaxed) == -1) {
 		return NH_ERR_ARGUMENT;
 	}
 	t.kind		 = -1;

@@ -17,13 +17,14 @@ int main(int argc, char** argv) {
 	const size_t head = base.size() < 1024 ? base.size() : 1024;
 	for (int it = 0; it < iters; ++it) {
 		std::vector<unsigned char> b = base;
-		const int kind = rng() % 6;
+		const int kind = rng() % 7;
 		if (kind == 0) b.resize(rng() % (b.size() + 1));
 		else if (kind == 1) for (int j = 0, n = 1 + rng() % 4; j < n; ++j) b[rng() % head] = static_cast<unsigned char>(rng());
 		else if (kind == 2) { const size_t at = rng() % (head - 8); const unsigned long long v = (rng() % 4 == 0) ? ~0ull >> (rng() % 64) : rng(); memcpy(&b[at], &v, 8); }
 		else if (kind == 3) { const size_t at = rng() % (head - 4); const unsigned v = static_cast<unsigned>(rng() % 64); memcpy(&b[at], &v, 4); }
 		else if (kind == 4) { b[rng() % head] ^= 1u << (rng() % 8); b.resize(head + rng() % (b.size() - head + 1)); }
-		else { const size_t at = rng() % (head - 8); const unsigned long long v = b.size() + (rng() % 64) - 32; memcpy(&b[at], &v, 8); }
+		else if (kind == 5) { const size_t at = rng() % (head - 8); const unsigned long long v = b.size() + (rng() % 64) - 32; memcpy(&b[at], &v, 8); }
+		else { const size_t at = rng() % (head - 8); const unsigned long long v = 0ull - 32ull * (1 + rng() % 64); memcpy(&b[at], &v, 8); } // just below 2^64: an offset that wraps when added to the data start
 		const char* tmp = argc > 4 ? argv[4] : "/tmp/nh_fuzz.gguf";
 		FILE* f = fopen(tmp, "wb"); fwrite(b.data(), 1, b.size(), f); fclose(f);
 		nh_gguf* g = nullptr;
@@ -37,6 +38,7 @@ int main(int argc, char** argv) {
 			if (nh_gguf_tensor_at(g, i, &ti) == 0) {
 				nh_gguf_tensor_info tj;
 				sink += strlen(ti.name) + (nh_gguf_find_tensor(g, ti.name, &tj) == 0);
+				if (ti.file_offset < nh_gguf_data_offset(g)) { printf("iter %d: tensor %s starts before the data section (%llu < %llu)\n", it, ti.name, (unsigned long long)ti.file_offset, (unsigned long long)nh_gguf_data_offset(g)); return 1; }
 				if (ti.file_offset + ti.byte_size > b.size()) { printf("iter %d: tensor %s past the end of the file (%llu + %llu > %zu)\n", it, ti.name, (unsigned long long)ti.file_offset, (unsigned long long)ti.byte_size, b.size()); return 1; }
 			}
 		}

@@ -99,6 +99,16 @@ def test_fails_loudly_without_a_gpu():
     p = C.c_void_p()
     assert lib.nh_malloc(C.byref(p), 1024) == -4  # no device: an error, never a silent CPU path
     assert lib.nh_q8_0_prepare() == -4
+    # the row limit of the mat-mat follows the launch grid of the kernel that would run (checked before any device call):
+    # 32 rows per workgroup row on tiled operands, 128 on packed blocks
+    assert lib.nh_q8_0_gemm_tiled(None, None, None, 65535 * 32 + 1, 32, 128, None) == -5
+    assert lib.nh_q8_0_gemm_tiled(None, None, None, 65535 * 32, 32, 128, None) == -1
+    assert lib.nh_q8_0_gemm(None, None, None, 65535 * 128 + 1, 32, 128, None) == -5
+    assert lib.nh_q8_0_gemm(None, None, None, 65535 * 128, 32, 128, None) == -1
+    assert lib.nh_q8_0_last_error() == -4
+    # the status plumbing of the device-side reports needs no device
+    assert "another stream" in _lib.status_string(-10) and "bounded wait" in _lib.status_string(-11)
+    assert lib.nh_q8_0_debug_set_spin_limit(0) == -6 and lib.nh_q8_0_debug_set_spin_limit(1 << 20) == 0
     assert lib.nh_q8_0_quantize(0x1000, 0x2000, 1, 32, None) == -4
     with pytest.raises(_lib.Q8Error):
         _lib.check("nh_q8_0_quantize", lib.nh_q8_0_quantize(0x1000, 0x2000, 1, 32, None))

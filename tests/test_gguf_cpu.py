@@ -144,6 +144,14 @@ def test_rejects_malformed_files(gguf, oracle, tmp_path):
     p = str(tmp_path / "align0.gguf")
     W.write_gguf(p, [("general.alignment", W.U32, 48)], [("t", [32], 8, blocks)], alignment=48)
     assert status_of(p) == -8  # not a power of two
+    # an offset just below 2^64 wraps to a small file offset when added to the data start: the tensor would alias the header
+    p = str(tmp_path / "wrap.gguf")
+    W.write_gguf(p, [], [("t", [32], 8, blocks)])
+    raw = bytearray(open(p, "rb").read())
+    at = 24 + (8 + 1) + 4 + 8 + 4  # header, name, n_dims, one dim, type: the record's offset field
+    assert struct.unpack_from("<Q", raw, at)[0] == 0
+    struct.pack_into("<Q", raw, at, 2**64 - 64)  # data starts at byte 64 of this file: 64 + (2^64 - 64) = 0
+    assert status_of(variant("wrap_patched.gguf", bytes(raw))) == -8
     # a v2 file and a file with no tensors are fine
     p = str(tmp_path / "v2.gguf")
     W.write_gguf(p, [("a", W.U8, 5)], [("t", [32], 8, blocks)], version=2)

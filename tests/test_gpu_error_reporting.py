@@ -1,0 +1,75 @@
+"""GPU: failures inside a launch reach the host as a status.
+
+* A workgroup of the one-launch FFN that gives up waiting for another workgroup's data leaves NaN in y AND a sticky error
+  that the next nh_stream_sync returns (NH_ERR_DEVICE_TIMEOUT, once).  The wait is made to give up from the host, by lowering
+  the poll limit to 1: every kernel still runs to its end.
+* The per-GPU scratch serves one stream at a time: a K-split launch on a second stream while the first stream still has
+  work in flight is refused with NH_ERR_BUSY before anything is launched.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import REL_L2_TOL, rel_l2, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+NH_ERR_BUSY, NH_ERR_DEVICE_TIMEOUT = -10, -11
+
+
+def test_ffn_timeout_is_reported_by_the_next_sync(q8, oracle):
+    lib = q8._lib.lib()
+    k, n_ff = 4096, 14336
+    wg, wu, wd = (q8.tile(q8.fill_weight_blocks(s, n, kk), n, kk) for s, (n, kk) in enumerate([(n_ff, k), (n_ff, k), (k, n_ff)]))
+    x = q8.fill_activations(3, k)
+    stream = torch.cuda.current_stream().cuda_stream
+    good = q8.ffn(wg, wu, wd, x, n_ff, k, k)
+    assert lib.nh_stream_sync(stream) == 0 and bool(torch.isfinite(good).all())
+    try:
+        assert lib.nh_q8_0_debug_set_spin_limit(1) == 0
+        bad = q8.ffn(wg, wu, wd, x, n_ff, k, k)
+        assert lib.nh_stream_sync(stream) == NH_ERR_DEVICE_TIMEOUT  # the workgroups that found their activation missing said so
+        assert bool(torch.isnan(bad).any())
+        assert lib.nh_stream_sync(stream) == 0  # reported once
+        assert lib.nh_q8_0_last_error() == 0
+    finally:
+        assert lib.nh_q8_0_debug_set_spin_limit(1 << 20) == 0
+    again = q8.ffn(wg, wu, wd, x, n_ff, k, k)
+    assert lib.nh_stream_sync(stream) == 0
+    assert np.array_equal(to_host(again), to_host(good))
+    assert "bounded wait" in q8._lib.status_string(NH_ERR_DEVICE_TIMEOUT)
+    assert lib.nh_q8_0_debug_set_spin_limit(0) == -6
+
+
+def test_scratch_in_use_on_another_stream_is_refused(q8, oracle):
+    lib = q8._lib.lib()
+    n, k = 4096, 14336  # K split over four workgroups per strip: the hand-off goes through the per-GPU scratch
+    w = oracle.fill_weights(5, n, k)
+    x = oracle.fill_activations(5, k)
+    wt, xd = q8.tile(to_dev(w), n, k), to_dev(x)
+    y_a = torch.empty(n, dtype=torch.float32, device="cuda")
+    y_b = torch.full((n,), 7.0, dtype=torch.float32, device="cuda")
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for _ in range(300):  # a few milliseconds of work on stream a
+        assert lib.nh_q8_0_gemv_tiled_f32(wt.data_ptr(), xd.data_ptr(), y_a.data_ptr(), n, k, a.cuda_stream) == 0
+    rc = lib.nh_q8_0_gemv_tiled_f32(wt.data_ptr(), xd.data_ptr(), y_b.data_ptr(), n, k, b.cuda_stream)
+    assert rc == NH_ERR_BUSY, rc
+    a.synchronize()
+    b.synchronize()
+    assert bool((y_b == 7.0).all())  # nothing was launched
+    # once stream a has drained the same call goes through, and both results are right
+    assert lib.nh_q8_0_gemv_tiled_f32(wt.data_ptr(), xd.data_ptr(), y_b.data_ptr(), n, k, b.cuda_stream) == 0
+    b.synchronize()
+    want = oracle.gemv(w, oracle.quantize_rows(x)[0], n, k)
+    assert rel_l2(to_host(y_a), want) <= REL_L2_TOL and np.array_equal(to_host(y_a), to_host(y_b))
+    assert "another stream" in q8._lib.status_string(NH_ERR_BUSY)
+    # the same stream twice in a row is the normal case and never refused; a shape without a K split does not touch the scratch
+    n2, k2 = 14336, 4096
+    w2 = q8.tile(q8.fill_weight_blocks(9, n2, k2), n2, k2)
+    x2 = q8.fill_activations(9, k2)
+    y2 = torch.empty(n2, dtype=torch.float32, device="cuda")
+    for _ in range(100):
+        assert lib.nh_q8_0_gemv_tiled_f32(wt.data_ptr(), xd.data_ptr(), y_a.data_ptr(), n, k, a.cuda_stream) == 0
+    assert lib.nh_q8_0_gemv_tiled_f32(w2.data_ptr(), x2.data_ptr(), y2.data_ptr(), n2, k2, b.cuda_stream) == 0
+    torch.cuda.synchronize()
