@@ -3,17 +3,18 @@
 
 Workload (the configuration the metric is quoted on): the LLaMA-3-8B FFN decode mat-vecs at batch 1 --
 gate and up, Q8_0 W [14336 x 4096], and down, Q8_0 W [4096 x 14336] -- with the activation quantize inside
-the step.  One step = quantize(x[4096]) -> gate, up ; quantize(h[14336]) -> down, enqueued by one native
-batch call.  The three mat-vecs of this configuration are independent (each has its own seeded input), which the
-batch runner sees from their input and output ranges, so it runs them as ONE launch of the grouped mat-vec kernel
-(every matrix cut as its own launch would cut it, the quantize inside the kernel).  The default run also reports the
-same step as two launches (gate+up, then down: what a caller gets who marks the down projection as ordered after
-the others) and as the one-launch FFN with the real dependency inside (down fed by SiLU(gate) * up).  Steps rotate over `--layers` distinct weight sets (default 16 x 187 MB = 3 GB) so that every
+the step.  The headline step is the form a model runs: down is fed by SiLU(gate) * up, all three mat-vecs, the activation
+quantizes and SiLU * up as ONE launch (nh_q8_0_ffn_f32).  The default run also reports the same three matrices as the
+configuration words them -- three mat-vecs with their own resident inputs, which the batch runner proves independent and
+groups into one launch (`ffn_grouped_independent`) -- and as two launches with the down projection ordered behind the
+others (`ffn_two_launches`); the single mat-vec of the first benchmark configuration ([4096 x 4096]) and the other decode
+shapes, cold (weights rotated through HBM) and cache-resident (`gemv_shapes`); the prefill mat-mat against the int8-MFMA
+roofline (`prefill`); and the whole-token decode leg (`decode`).  Steps rotate over `--layers` distinct weight sets (default 16 x 187 MB = 3 GB) so that every
 byte comes from HBM and not from the 256 MB last-level cache.  Inputs are resident in HBM before the timed
 region; synthetic data from the library's counter-based generator (seed 0).
 
 Prints ONE JSON line.  `value` = algorithmic bytes per step / wall time per step.  `roofline` is for the
-dominant kernel (the grouped mat-vec): algorithmic bytes per launch / its average duration, measured live with
+dominant kernel (the one-launch FFN): algorithmic bytes per launch / its average duration, measured live with
 start/stop timestamps carried in each launch's own dispatch packet.  `cpu_baseline` is the AVX2 restatement
 of the reference arithmetic on the host's cores (a reported number, not the target).
 """
@@ -33,8 +34,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 GATE_N, HIDDEN, FFN = 14336, 4096, 14336
 # HBM bytes per launch of the dominant kernel (mean over the step's launches): FETCH_SIZE and WRITE_SIZE from two
 # rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for a plain 64 MiB copy
-# (FETCH_SIZE x 1.99927, WRITE_SIZE x 1.0).  A hardware-counter figure cannot be taken live; this is the recorded one.
-# Keyed by --ffn-mode; None = not measured yet for that mode.
+# (FETCH_SIZE x 1.99927, WRITE_SIZE x 1.0).  A hardware-counter figure cannot be taken live; this is the recorded one
+# (the JSON line says so in roofline.traffic_source).  Keyed by --ffn-mode; None = not measured yet for that mode.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"group": 188267907, "two": 94168857, "fused": 188120789}
 
 
@@ -67,11 +68,12 @@ def main() -> int:
     ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover", "llama70b", "f32act"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
-    ap.add_argument("--ffn-mode", choices=["group", "two", "fused"], default="group",
-                    help="group (default): the step's three mat-vecs through nh_q8_0_mul_mat_batch, the down projection fed from a resident fp32 "
-                    "vector (mat-vecs only, as the metric is defined); the runner finds them independent and issues one grouped launch.  two: the same "
-                    "with the down projection marked ordered: gate+up, then down, two launches.  fused: the step as one launch with the real "
-                    "dependency inside (nh_q8_0_ffn_f32: gate, up, SiLU*up, down).  The default run reports the other two beside the headline")
+    ap.add_argument("--ffn-mode", choices=["group", "two", "fused"], default="fused",
+                    help="fused (default): the step as one launch with the real dependency inside (nh_q8_0_ffn_f32: gate, up, SiLU*up, down).  "
+                    "group: the step's three mat-vecs through nh_q8_0_mul_mat_batch, the down projection fed from a resident fp32 vector; the "
+                    "runner finds them independent and issues one grouped launch.  two: the same with the down projection marked ordered: "
+                    "gate+up, then down, two launches.  The default run reports the other two beside the headline")
+    ap.add_argument("--no-extras", action="store_true", help="skip the per-shape mat-vec figures and the prefill leg (for profiler runs)")
     ap.add_argument("--no-decode", action="store_true", help="skip the whole-model decode-step leg (8 GB of weights)")
     ap.add_argument("--decode-tokens", type=int, default=200, help="timed tokens of the decode-step leg")
     ap.add_argument("--roofline-steps", type=int, default=0, help="steps of the per-kernel timing pass (default: min(steps, 1000))")
@@ -230,6 +232,8 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH[mode],
+            "traffic_source": "recorded from two rocprofv3 --pmc runs of this command (FETCH_SIZE, WRITE_SIZE, scaled by a plain 64 MiB copy; summary under profiles/): "
+                              "hardware counters cannot be read inside this run",
             "bytes_per_launch": launch_bytes,
             "avg_launch_us": round(avg_ms * 1e3, 3),
             "min_launch_us": round(mn.value * 1e3, 3),
@@ -238,11 +242,11 @@ def main() -> int:
         },
     }
 
-    if mode == "group":
+    if mode == "fused":
         # the same step the other two ways, timed the same way, beside the headline
         def timed_other(m: str) -> tuple[float, bool]:
             nonlocal fused
-            fused = m == "fused"
+            fused = False
             set_ordered(1 if m == "two" else 0)
             run_steps(args.warmup)
             torch.cuda.synchronize()
@@ -251,11 +255,12 @@ def main() -> int:
             torch.cuda.synchronize()
             sec = (time.perf_counter() - t) / args.steps
             ok = bool(torch.isfinite(y_down).all())
-            fused = False
+            fused = True
             set_ordered(0)
             return sec, ok
 
-        for m, key, entry in (("two", "ffn_two_launches", "nh_q8_0_mul_mat_batch, down marked ordered"), ("fused", "ffn_one_launch", "nh_q8_0_ffn_f32")):
+        for m, key, entry in (("two", "ffn_two_launches", "nh_q8_0_mul_mat_batch, down marked ordered (its input a resident vector)"),
+                              ("group", "ffn_grouped_independent", "nh_q8_0_mul_mat_batch, the three mat-vecs with their own resident inputs, proved independent and grouped into one launch")):
             sec, ok = timed_other(m)
             nb = sum(launch_bytes_of(m))
             result[key] = {"entry": entry, "ms_per_step": round(sec * 1e3, 6), "GBs": round(nb / sec / 1e9, 1), "pct_of_hbm_peak": round(100.0 * nb / sec / 1e9 / HBM_PEAK_GBS, 2),
@@ -263,6 +268,11 @@ def main() -> int:
 
     del layers, op_lists
     torch.cuda.empty_cache()
+    if not args.no_extras:
+        result["gemv_shapes"] = gemv_shapes(min(args.steps, 400))
+        pre = side_workload("prefill", 100, 10)
+        result["prefill"] = {"metric": pre["metric"], "value": pre["value"], "unit": pre["unit"], "ms_per_step": pre["ms_per_step"], "config": pre["config"], "roofline": pre["roofline"]}
+        torch.cuda.empty_cache()
     if not args.no_decode:
         result["decode"] = decode_step(args.decode_tokens)
 
@@ -271,6 +281,63 @@ def main() -> int:
 
     print(json.dumps(result))
     return 0
+
+
+def gemv_shapes(steps: int) -> dict:
+    """One fused quantize + mat-vec launch per step at the decode shapes of the benchmark configurations, each timed twice:
+    `cold` rotates over enough weight copies that every launch streams its matrix from HBM (> 512 MB in rotation), `hot`
+    repeats one copy (cache-resident when the matrix fits the 256 MB last-level cache: a latency figure, not an HBM one).
+    Per-launch kernel time from the dispatch packets' own timestamps; GB/s = algorithmic bytes / kernel time."""
+    import torch
+
+    from nihilus_amd import _lib, q8_0
+
+    lib = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    shapes = [("config1_4096x4096", [4096], 4096), ("down_4096x14336", [4096], 14336), ("gate_14336x4096", [14336], 4096), ("qkv_6144x4096", [4096, 1024, 1024], 4096),
+              ("o_4096x4096", [4096], 4096), ("kv_1024x4096", [1024], 4096), ("lm_head_128256x4096", [128256], 4096)]
+    out = {}
+    seed = 30
+    for name, ns, k in shapes:
+        wbytes = sum(weight_bytes(n, k) for n in ns)
+        copies = max(2, min(32, int(6.0e8 // wbytes) + 1))
+        sets = []
+        for _ in range(copies):
+            mats = []
+            for n in ns:
+                b = q8_0.fill_weight_blocks(seed, n, k)
+                seed += 1
+                mats.append(q8_0.tile(b, n, k))
+                del b
+            sets.append(mats)
+        x = q8_0.fill_activations(seed, k)
+        ys = [torch.empty(n, dtype=torch.float32, device=x.device) for n in ns]
+        cnt = len(ns)
+        yp, np_ = (C.c_void_p * cnt)(*[y.data_ptr() for y in ys]), (C.c_int64 * cnt)(*ns)
+        wps = [(C.c_void_p * cnt)(*[w.data_ptr() for w in mats]) for mats in sets]
+        nbytes = fused_launch_bytes(ns, k)
+
+        def run(i, rotate):
+            rc = lib.nh_q8_0_gemv_tiled_multi_f32(wps[i % copies if rotate else 0], yp, np_, cnt, x.data_ptr(), k, stream)
+            if rc != 0:
+                _lib.check("nh_q8_0_gemv_tiled_multi_f32", rc)
+
+        row = {"bytes_per_launch": nbytes, "weight_copies_rotated": copies}
+        for label, rotate in (("cold", True), ("hot", False)):
+            for i in range(20):
+                run(i, rotate)
+            torch.cuda.synchronize()
+            _lib.check("nh_profile_begin", lib.nh_profile_begin(1, steps))
+            for i in range(steps):
+                run(i, rotate)
+            tot, n_l, mn, mx = C.c_double(), C.c_int64(), C.c_double(), C.c_double()
+            _lib.check("nh_profile_end", lib.nh_profile_end(C.byref(tot), C.byref(n_l), C.byref(mn), C.byref(mx)))
+            us = tot.value / max(1, n_l.value) * 1e3
+            row[label] = {"avg_launch_us": round(us, 3), "GBs": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        out[name] = row
+        del sets, wps
+        torch.cuda.empty_cache()
+    return out
 
 
 INT8_MFMA_PEAK_TOPS = 5033.0  # MI355X published dense int8 matrix rate
@@ -618,24 +685,26 @@ def cpu_baseline(budget_s: float) -> dict:
     import oracle as O  # the checker, used here only as the reported CPU baseline
 
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
-    threads = max(1, min(16, cores))  # the GPU box gives one job 16 cores' worth of CPU
+    # every core this job may use, up to 16: a one-GPU job on the benchmark host is given 16 cores' worth of CPU whatever the
+    # machine reports, and more threads than that only queue.  Workers are pinned one per core (cpu/thread_pool.hpp:34-56 does).
+    threads = max(1, min(16, cores))
     n_sets = 8  # 0.5 GB per shape: well past the host's last-level cache
     w_gate = np.concatenate([O.fill_weights(0, GATE_N, HIDDEN, first_block=i * GATE_N * (HIDDEN // 32)) for i in range(n_sets)])
     w_down = np.concatenate([O.fill_weights(7, HIDDEN, FFN, first_block=i * HIDDEN * (FFN // 32)) for i in range(n_sets)])
     x = O.fill_activations(0, HIDDEN)
     h = O.fill_activations(1, FFN)
     # short calibration, then a bounded sample
-    t_g = O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, threads, 3, pin=False)
-    t_d = O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, threads, 3, pin=False)
+    t_g = O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, threads, 3, pin=True)
+    t_d = O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, threads, 3, pin=True)
     per_pass = 2 * t_g + t_d
     passes = int(max(3, min(400, budget_s / max(per_pass, 1e-6))))
-    t_g = O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, threads, 2 * passes, pin=False)
-    t_d = O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, threads, passes, pin=False)
+    t_g = O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, threads, 2 * passes, pin=True)
+    t_d = O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, threads, passes, pin=True)
     sec = 2 * t_g + t_d
     nbytes = 2 * cpu_gemv_bytes(GATE_N, HIDDEN) + cpu_gemv_bytes(HIDDEN, FFN)
     # the same step on one thread (a few passes: ~10 ms each)
     one_passes = int(max(2, min(passes, 2.0 / max(sec * threads, 1e-6))))  # about two seconds
-    sec_1 = 2 * O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, 1, 2 * one_passes, pin=False) + O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, 1, one_passes, pin=False)
+    sec_1 = 2 * O.time_gemv_avx2(w_gate, n_sets, x, GATE_N, HIDDEN, 1, 2 * one_passes, pin=True) + O.time_gemv_avx2(w_down, n_sets, h, HIDDEN, FFN, 1, one_passes, pin=True)
     model = ""
     try:
         with open("/proc/cpuinfo") as f:
@@ -651,7 +720,7 @@ def cpu_baseline(budget_s: float) -> dict:
         "cores": threads,
         "kind": "port",
         "sample": f"{passes} passes of the same FFN step (gate, up, down mat-vecs + quantize) over {n_sets} rotating weight sets, "
-        f"AVX2/FMA/F16C restatement of the reference arithmetic, {threads} threads, rows claimed through an atomic chunk counter",
+        f"AVX2/FMA/F16C restatement of the reference arithmetic, {threads} pinned threads ({cores} cores visible to the job, at most 16 used), rows claimed through an atomic chunk counter",
         "cpu_model": model,
         "ms_per_step": round(sec * 1e3, 3),
         "single_thread": {"value": round(nbytes / sec_1 / 1e9, 2), "unit": "GB/s", "cores": 1, "ms_per_step": round(sec_1 * 1e3, 3), "passes": one_passes},

@@ -162,6 +162,11 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 			}
 			if (++spins >= spin_limit) {
 				timed_out = true;
+				// tell the host (an ordinary vector store to pinned host memory).  Done here, not where the NaN is set: kept for
+				// the end of the function the pointer and the branch cost the hot path 25 registers
+				if (lane == 0 && dump) {
+					__hip_atomic_store(static_cast<unsigned*>(dump), static_cast<unsigned>(DEVICE_ERROR_PUBLISH_TIMEOUT), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+				}
 				break;
 			}
 			__builtin_amdgcn_s_sleep(8);
@@ -285,10 +290,7 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	}
 	if constexpr (XMODE == X_PUBLISHED) {
 		if (timed_out) {
-			acc = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output ...
-			if (lane == 0 && dump) { // ... and to the host (an ordinary vector store to pinned host memory)
-				__hip_atomic_store(static_cast<unsigned*>(dump), static_cast<unsigned>(DEVICE_ERROR_PUBLISH_TIMEOUT), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-			}
+			acc = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output as well
 		}
 	}
 	return acc;

@@ -137,6 +137,21 @@ float nha_vec_dot_q8_0_q8_0_x16(int64_t n_blocks, const void* vx, const void* vy
 
 /* ------------------------------------------------------------------ threaded GEMV / GEMM */
 
+/* The t-th CPU of the mask this process may run on (a job is often confined to a subset of the machine's cores, so "core t"
+ * is not a valid target in general); -1 if the mask holds fewer. */
+static int nth_allowed_cpu(int t) {
+	cpu_set_t set;
+	if (sched_getaffinity(0, sizeof(set), &set) != 0) {
+		return -1;
+	}
+	for (int c = 0; c < CPU_SETSIZE; ++c) {
+		if (CPU_ISSET(c, &set) && t-- == 0) {
+			return c;
+		}
+	}
+	return -1;
+}
+
 typedef struct {
 	const uint8_t* w;
 	const uint8_t* aq;
@@ -188,7 +203,7 @@ int nha_gemm_q8_0_mt(const void* w, const void* aq, float* c, int64_t m_rows, in
 	job_t* jobs	   = (job_t*)malloc(sizeof(job_t) * (size_t)threads);
 	pthread_t* tid = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)threads);
 	for (int t = 0; t < threads; ++t) {
-		jobs[t] = (job_t){ (const uint8_t*)w, (const uint8_t*)aq, c, m_rows, n_rows, nb, 16, &next, pin ? t : -1 };
+		jobs[t] = (job_t){ (const uint8_t*)w, (const uint8_t*)aq, c, m_rows, n_rows, nb, 16, &next, pin ? nth_allowed_cpu(t) : -1 };
 	}
 	for (int t = 0; t < threads; ++t) { /* the caller's own thread is left alone so its affinity is never changed */
 		pthread_create(&tid[t], 0, worker, &jobs[t]);
@@ -268,7 +283,7 @@ double nha_time_gemv(const void* w_all, int64_t n_mats, const float* x, float* y
 	tjob_t* jobs   = (tjob_t*)malloc(sizeof(tjob_t) * (size_t)threads);
 	pthread_t* tid = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)threads);
 	for (int t = 0; t < threads; ++t) {
-		jobs[t] = (tjob_t){ (const uint8_t*)w_all, n_mats, n_rows * nb * BLK, x, xq, y, n_rows, k, nb, iters, counters, &bar, t, pin ? t : -1 };
+		jobs[t] = (tjob_t){ (const uint8_t*)w_all, n_mats, n_rows * nb * BLK, x, xq, y, n_rows, k, nb, iters, counters, &bar, t, pin ? nth_allowed_cpu(t) : -1 };
 	}
 	struct timespec t0, t1;
 	clock_gettime(CLOCK_MONOTONIC, &t0);
