@@ -36,7 +36,7 @@ GATE_N, HIDDEN, FFN = 14336, 4096, 14336
 # rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for a plain 64 MiB copy
 # (FETCH_SIZE x 1.99927, WRITE_SIZE x 1.0).  A hardware-counter figure cannot be taken live; this is the recorded one
 # (the JSON line says so in roofline.traffic_source).  Keyed by --ffn-mode; None = not measured yet for that mode.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"group": 188267907, "two": 94168857, "fused": 188120789}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"group": 188264835, "two": 94169420, "fused": 188130005}
 
 
 def weight_bytes(n: int, k: int) -> int:
