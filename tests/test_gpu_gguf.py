@@ -42,16 +42,19 @@ def test_upload_errors(q8, oracle, tmp_path):
     from nihilus_amd import gguf as G
 
     path = str(tmp_path / "e.gguf")
-    W.write_gguf(path, [], [("a", [96, 4], 8, oracle.fill_weights(1, 4, 96).tobytes()), ("b", [128], 0, W.f32_bytes(np.zeros(128)))])
+    W.write_gguf(path, [], [("a", [96, 4], 8, oracle.fill_weights(1, 4, 96).tobytes()), ("b", [128], 0, W.f32_bytes(np.zeros(128))),
+                               ("c", [128, 4], 8, oracle.fill_weights(2, 4, 128).tobytes())])
     lib = _lib.lib()
     with G.GGUFFile(path) as f:
-        a, b = f.find("a"), f.find("b")
+        a, b, c = f.find("a"), f.find("b"), f.find("c")
         dst = torch.zeros(8192, dtype=torch.uint8, device="cuda")
         st = torch.zeros(8192, dtype=torch.uint8, device="cuda")
         up = lambda info, tiled, staging, n: lib.nh_gguf_upload_tensor(f._h, C.byref(info), dst.data_ptr(), tiled, staging, n, None)
         assert up(a, 1, st.data_ptr(), 8192) == -3  # K = 96 is not a multiple of 128
         assert up(b, 1, st.data_ptr(), 8192) == -6  # not Q8_0
         assert up(a, 0, None, 0) == 0
-        a.dims[0] = 128  # pretend: staging checks come next
-        assert up(a, 1, None, 0) == -1
-        assert up(a, 1, st.data_ptr(), 10) == -6
+        assert up(c, 1, None, 0) == -1
+        assert up(c, 1, st.data_ptr(), 10) == -6
+        assert up(c, 1, st.data_ptr(), 8192) == 0
+        a.dims[0] = 128  # a record edited by the caller no longer matches its byte size
+        assert up(a, 1, st.data_ptr(), 8192) == -6
