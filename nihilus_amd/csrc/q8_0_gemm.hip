@@ -23,6 +23,7 @@ constexpr int GEMM_TN	   = 2; // along N
 constexpr int GEMM_BM	   = GEMM_WAVES_M * GEMM_TM * 32; // 128
 constexpr int GEMM_BN	   = GEMM_WAVES_N * GEMM_TN * 32; // 128
 constexpr int GEMM_THREADS = GEMM_WAVES_M * GEMM_WAVES_N * 64;
+constexpr int GEMM_STREAM_TILE_MIN_COLUMN_BLOCKS = 192; // 128-row column blocks from which the tile kernel also takes the few-row (batched decode) shapes
 
 // 16 operand bytes for (row strip, block b): lane supplies row strip*32 + lane%32, half lane/32.
 template<bool TILED> __device__ __forceinline__ v4i load_operand(const uint8_t* base, int rows, int nb, int strip, int b, int lane) {
@@ -151,9 +152,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const uint8_t* __res
 //
 // Both operands carry a scale per 32-quant block, so each 32x32x32 int8 MFMA result (1024 exact block sums, 16 per
 // lane) has to be converted and folded into the fp32 accumulator before the next block: 16 conversions + 16
-// multiply-adds per lane per MFMA.  Measured on this part, a SIMD retires one wave64 VALU instruction per ~2.4 cycles
-// once it holds two or more waves (a lone wave issues one per ~5), and MFMA and VALU work does not overlap: a
-// (tile, block) costs 32 + 32 matrix-pipe cycles plus 32 x 2.4 VALU cycles, ~141 cycles against the 32 of the int8
+// multiply-adds per lane per MFMA.  Measured on this part, a SIMD retires one wave64 VALU instruction per ~2.5 cycles
+// once it holds two or more waves (a lone wave issues one per ~4-5), and MFMA and VALU time add on a SIMD, also across
+// waves: a (tile, block) costs 32 + 32 matrix-pipe cycles plus 32 x 2.5 VALU cycles, ~145 cycles against the 32 of the int8
 // MFMA alone.  That is the ceiling (~22 % of the int8 MFMA peak); the kernel is shaped to add as little as possible:
 //   * the scale products f32(dA[m][b]) * f32(dW[n][b]) are formed on the matrix pipe: one v_mfma_f32_32x32x8_f16 whose
 //     operands are the two blocks' fp16 scales as stored, each in the k = 0 slot ({d, 0, 0, 0}; lanes 32..63 supply
@@ -165,20 +166,41 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const uint8_t* __res
 //     TM activation strips, copied global -> LDS one group ahead (double-buffered, one barrier per group, the copy
 //     spread over the four waves) and read back as conflict-free 16-byte-per-lane operand images plus one half-word
 //     read per scale;
+//   * every global address is a wave-uniform base in scalar registers plus a 32-bit lane offset (the addressing mode of
+//     global_load with a scalar base): no 64-bit address arithmetic on the VALU, which is the pipe the fold saturates,
+//     and ~10 fewer registers than per-lane pointers (the difference between spilling and not at two activation strips);
 //   * latency is hidden by occupancy, not by a software pipeline: one result-register set per tile keeps the kernel
 //     at <= 128 VGPRs, four workgroups per CU, four waves per SIMD.  (A two-result-set, software-pipelined variant
 //     at two waves per SIMD measured 8 % slower: with so few waves the SIMD falls back to the lone-wave issue rate
 //     whenever one of them waits.)
-template<int TM, bool DUMP, int KS = 1>
+// a 64-bit offset that the compiler may keep in scalar registers (it is the same for every lane of the wave)
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+	const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v)), hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(static_cast<uint64_t>(v) >> 32));
+	return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+typedef const __attribute__((address_space(1))) uint8_t* gptr_u8;
+// base + wave-uniform offset as a pointer the compiler must keep in scalar registers (and cannot fold the lane offset into)
+__device__ __forceinline__ gptr_u8 scalar_base(const uint8_t* base, int64_t uniform_off) {
+	gptr_u8 p = (gptr_u8)(base) + uniform_off;
+	asm volatile("" : "+s"(p));
+	return p;
+}
+template<typename T, bool NT> __device__ __forceinline__ T load_sv(gptr_u8 p, uint32_t lane_off) {
+	typedef const __attribute__((address_space(1))) T* gp;
+	if constexpr (NT) {
+		return __builtin_nontemporal_load(reinterpret_cast<gp>(p + lane_off));
+	} else {
+		return *reinterpret_cast<gp>(p + lane_off);
+	}
+}
+
+template<int TM, bool DUMP, int KS = 1, bool STREAM = false>
 __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* C, const float* R, int32_t* __restrict__ sums, int M, int N,
 	int groups) {
 	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
 	constexpr int STAGE_BYTES = DATA_BYTES + 16;
-	// KS > 1: the workgroup holds KS sets of four waves; set kr walks groups [kr * groups / KS, (kr + 1) * groups / KS) with its
-	// own activation stages, and the sets' results are added to the first's through LDS at the end (set order, fixed).  A
-	// grid too small to give every SIMD its four waves gets them this way without a second pass over memory.
-	__shared__ __align__(16) uint8_t lds_all[KS][2 * STAGE_BYTES];
-	__shared__ float red[KS > 1 ? 4 * TM * 16 * 64 : 1];
+	__shared__ __align__(16) uint8_t lds_all[KS][2 * STAGE_BYTES + 256]; // + 256: where waves that copy no scale table put theirs
 	typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 	typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -198,44 +220,41 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	if ((tid & 255) < 8) {
 		*reinterpret_cast<uint32_t*>(lds + ((tid & 255) >> 2) * STAGE_BYTES + DATA_BYTES + 4 * (tid & 3)) = 0u;
 	}
-	const uint8_t* w_src = W + macro_offset(min(ns, n_strips - 1), g_base, groups);
+	// every address below is a wave-uniform part (scalar registers, advanced by scalar adds) plus one of three lane constants
+	const uint32_t lane16 = 16u * lane, lane4 = 4u * lane, sc8 = 8u * (lane & 31);
+	const int64_t w_off	  = uniform_i64(macro_offset(min(ns, n_strips - 1), g_base, groups));
 	struct w_regs {
 		v4i q[GROUP_BLOCKS];
 		v2u d;
 	};
-	auto fetch_w = [&](int g, w_regs& r) {
-		const uint8_t* p = w_src + static_cast<int64_t>(g) * MACRO_BYTES;
-#pragma unroll
-		for (int k = 0; k < GROUP_BLOCKS; ++k) {
-			r.q[k] = *reinterpret_cast<const v4i*>(p + k * TILE_BYTES + 16 * lane);
-		}
-		r.d = *reinterpret_cast<const v2u*>(p + MACRO_D_OFFSET + 8 * (lane & 31));
-	};
 	// activations: global -> registers -> LDS, shared out over the four waves: wave w moves tiles TM*w .. TM*w+TM-1 of the
 	// TM*4 tiles of a group, waves 0..TM-1 also the 256-byte scale table of strip w
-	const uint8_t* a_src[TM];
-	int a_dst[TM];
+	int64_t a_off[TM];
+	uint32_t a_dst[TM];
 #pragma unroll
 	for (int j = 0; j < TM; ++j) {
 		const int u = TM * wave + j;
-		a_src[j]	= A + macro_offset(min(ms0 + u / 4, m_strips - 1), g_base, groups) + (u % 4) * TILE_BYTES + 16 * lane;
-		a_dst[j]	= (u / 4) * MACRO_BYTES + (u % 4) * TILE_BYTES + 16 * lane;
+		a_off[j]	= uniform_i64(macro_offset(min(ms0 + u / 4, m_strips - 1), g_base, groups) + (u % 4) * TILE_BYTES);
+		a_dst[j]	= (u / 4) * MACRO_BYTES + (u % 4) * TILE_BYTES + lane16;
 	}
-	const bool sc_copier   = wave < TM;
-	const uint8_t* sc_src = A + macro_offset(min(ms0 + min(wave, TM - 1), m_strips - 1), g_base, groups) + MACRO_D_OFFSET + 4 * lane;
-	const int sc_dst	   = min(wave, TM - 1) * MACRO_BYTES + MACRO_D_OFFSET + 4 * lane;
+	// every wave copies a dword per lane of a scale table (waves >= TM: strip TM-1's again, stored nowhere), so that all waves
+	// issue the same loads
+	const int64_t sc_off  = uniform_i64(macro_offset(min(ms0 + min(wave, TM - 1), m_strips - 1), g_base, groups) + MACRO_D_OFFSET);
+	const uint32_t sc_dst = wave < TM ? wave * MACRO_BYTES + MACRO_D_OFFSET + lane4 : 2 * STAGE_BYTES + lane4;
+	const uint32_t sc_stage = wave < TM ? STAGE_BYTES : 0; // the spare area is not staged
 	struct a_regs {
 		v4i q[TM];
 		uint32_t d;
 	};
 	auto fetch_a = [&](int g, a_regs& r) {
+		const int64_t adv = static_cast<int64_t>(g) * MACRO_BYTES;
+		uint32_t l16 = lane16, l4 = lane4;
+		asm volatile("" : "+v"(l16), "+v"(l4));
 #pragma unroll
 		for (int j = 0; j < TM; ++j) {
-			r.q[j] = *reinterpret_cast<const v4i*>(a_src[j] + static_cast<int64_t>(g) * MACRO_BYTES);
+			r.q[j] = load_sv<v4i, false>(scalar_base(A, a_off[j] + adv), l16);
 		}
-		if (sc_copier) {
-			r.d = *reinterpret_cast<const uint32_t*>(sc_src + static_cast<int64_t>(g) * MACRO_BYTES);
-		}
+		r.d = load_sv<uint32_t, false>(scalar_base(A, sc_off + adv), l4);
 	};
 	auto stash_a = [&](int stage, const a_regs& r) {
 		uint8_t* p = lds + stage * STAGE_BYTES;
@@ -243,9 +262,18 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		for (int j = 0; j < TM; ++j) {
 			*reinterpret_cast<v4i*>(p + a_dst[j]) = r.q[j];
 		}
-		if (sc_copier) {
-			*reinterpret_cast<uint32_t*>(p + sc_dst) = r.d;
+		*reinterpret_cast<uint32_t*>(lds + stage * sc_stage + sc_dst) = r.d;
+	};
+	auto fetch_w = [&](int g, w_regs& r) {
+		const int64_t at = w_off + static_cast<int64_t>(g) * MACRO_BYTES;
+		const gptr_u8 p	 = scalar_base(W, at);
+		uint32_t l16 = lane16, l8 = sc8;
+		asm volatile("" : "+v"(l16), "+v"(l8)); // the widening of a lane offset has to stay beside its loads for scalar base + 32-bit lane offset to be picked as the addressing mode
+#pragma unroll
+		for (int k = 0; k < GROUP_BLOCKS; ++k) {
+			r.q[k] = load_sv<v4i, STREAM>(p + k * TILE_BYTES, l16);
 		}
+		r.d = load_sv<v2u, STREAM>(scalar_base(W, at + MACRO_D_OFFSET), l8);
 	};
 	v16f acc[TM];
 #pragma unroll
@@ -253,19 +281,23 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		acc[i] = v16f{ 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
 	}
 	const int a_sc_rel = half ? DATA_BYTES : MACRO_D_OFFSET + 8 * (lane & 31);
+	const int last	   = g_len - 1;
 
 	w_regs wa, wb;
 	a_regs pre;
-	fetch_w(0, wa);
 	fetch_a(0, pre);
+	fetch_w(0, wa);
 	stash_a(0, pre);
 	__syncthreads();
+	// One trip = one 128-quant group.  Requested at its start: the next group's activation tiles, then its weight tiles -- in
+	// that order, because loads return in issue order: the (cached) activations are needed at the trip's end, for the barrier,
+	// and must not queue behind weights that have until the next trip to arrive.  Past the end the last group is requested
+	// again (a cache hit that nobody uses): every trip issues the same loads, so every wait the compiler places is a count
+	// (a load under a condition makes it wait for everything outstanding instead).
 	auto trip = [&](int g, w_regs& cur, w_regs& nxt) {
-		const bool more = g + 1 < g_len;
-		if (more) {
-			fetch_w(g + 1, nxt);
-			fetch_a(g + 1, pre);
-		}
+		fetch_a(min(g + 1, last), pre);
+		fetch_w(min(g + 1, last), nxt);
+		__builtin_amdgcn_sched_barrier(0);
 		if (half) {
 			cur.d = v2u{ 0u, 0u };
 		}
@@ -301,9 +333,7 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 				}
 			}
 		}
-		if (more) {
-			stash_a((g + 1) & 1, pre);
-		}
+		stash_a((g + 1) & 1, pre);
 		__syncthreads();
 	};
 	for (int g = 0; g < g_len; g += 2) {
@@ -314,7 +344,9 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	}
 	if constexpr (KS > 1 && !DUMP) {
 		// sets 1 .. KS-1 park their tiles one after the other in the same LDS buffer, set 0 adds them (set order, fixed)
-		float* slot = red + wave * (TM * 16 * 64);
+		static_assert(sizeof(lds_all) >= 4 * TM * 16 * 64 * sizeof(float), "the stages double as the reduction buffer");
+		__syncthreads(); // every set is through with its stages
+		float* slot = reinterpret_cast<float*>(&lds_all[0][0]) + wave * (TM * 16 * 64);
 #pragma unroll
 		for (int k = 1; k < KS; ++k) {
 			if (kr == k) {
@@ -360,7 +392,7 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	}
 }
 
-template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s) {
+template<int TM, bool STREAM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s) {
 	const int groups   = k / GROUP_K;
 	const int m_strips = (m + 31) / 32, n_strips = (n + 31) / 32;
 	const dim3 grid(static_cast<unsigned>((n_strips + 3) / 4), static_cast<unsigned>((m_strips + TM - 1) / TM));
@@ -374,26 +406,24 @@ template<int TM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const u
 		ks *= 2;
 	}
 	if (ks == 4) {
-		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4>, grid, dim3(1024), 0, s, w, a, C, R, sums, m, n, groups);
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4, STREAM>, grid, dim3(1024), 0, s, w, a, C, R, sums, m, n, groups);
 	}
 	if (ks == 2) {
-		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2>, grid, dim3(512), 0, s, w, a, C, R, sums, m, n, groups);
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2, STREAM>, grid, dim3(512), 0, s, w, a, C, R, sums, m, n, groups);
 	}
-	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false>, grid, dim3(256), 0, s, w, a, C, R, sums, m, n, groups);
+	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 1, STREAM>, grid, dim3(256), 0, s, w, a, C, R, sums, m, n, groups);
 }
 
-// Tile choice.  One wave alone issues a VALU instruction only every ~5 cycles (two or more per SIMD reach ~2.4), so
-// the grid must give every SIMD at least two waves: 64-row workgroup tiles (half the LDS and L2 traffic per MFMA) when
-// that still leaves >= 512 workgroups, 32-row tiles otherwise.
-static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s) {
+// Two activation strips per wave whenever there are two: every weight tile fetched is used twice, which halves what a CU
+// has to take in per MFMA (that intake, not the MFMA rate, bounds the one-strip form); the K sets give back the waves the
+// halved grid loses.  stream: the weights are read once and not again (a batch of decode rows against a large matrix), so
+// their loads bypass the caches.
+static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s, bool stream) {
 	const int64_t ms = (m + 31) / 32;
-	// Two activation strips per wave whenever there are two: every weight tile fetched is used twice, which halves what a CU
-	// has to take in per MFMA (that intake, not the MFMA rate, bounds the one-strip form); the K sets below give back the
-	// waves the halved grid loses.
-	if (ms >= 2) {
-		return launch_gemm_tiled_t<2>(w, a, C, R, sums, m, n, k, s);
+	if (stream) {
+		return ms >= 2 ? launch_gemm_tiled_t<2, true>(w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, true>(w, a, C, R, sums, m, n, k, s);
 	}
-	return launch_gemm_tiled_t<1>(w, a, C, R, sums, m, n, k, s);
+	return ms >= 2 ? launch_gemm_tiled_t<2, false>(w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, false>(w, a, C, R, sums, m, n, k, s);
 }
 
 __global__ void zero_c_kernel(float* c, const float* src, int64_t n) {
@@ -422,11 +452,21 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 		// 128-row x 32-row tiles that the tile kernel would leave most SIMDs with one wave or none (measured: it needs
 		// more than one workgroup per CU to pay): the same streaming kernel over groups of 64 rows, K split over the
 		// waves of a workgroup, the weights coming from cache after the first group.
-		const int64_t tile_workgroups = ((N + 127) / 128) * ((M + 31) / 32);
+		const int64_t column_blocks	  = (N + 127) / 128;
+		const int64_t tile_workgroups = column_blocks * ((M + 31) / 32);
+		// A matrix with enough 128-row column blocks to occupy the chip by itself takes the tile kernel at any M: its four
+		// waves share each activation tile through LDS, where the streaming kernel's eight waves fetch one each from L2 --
+		// at 32 to 64 rows that is one to two times the weight bytes in extra traffic into every CU, and what a CU can take
+		// in is what bounds both kernels ([28672 x 8192] at M = 16 / 32 / 64: 50 / 55 / 75 us streaming, 44 / 44 / 69 us
+		// here; [128256 x 8192]: 193 / - / 298 against 182 / - / 221 us).  Below that the tile kernel's grid leaves CUs idle
+		// ([14336 x 4096] at M = 64: 30 us against 23 us) and the streaming kernel, which can split K over workgroups, stays.
+		if (M <= GEMM_SKINNY_MAX_M && column_blocks >= GEMM_STREAM_TILE_MIN_COLUMN_BLOCKS) {
+			return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, true);
+		}
 		if (M <= GEMM_SKINNY_MAX_M || tile_workgroups <= 256) {
 			return launch_gemm_skinny(W, Aq, C, sums, M, N, K, s, residual);
 		}
-		return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s);
+		return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, false);
 	} else {
 		if (sums) {
 			gemm_kernel<false, true><<<grid, dim3(GEMM_THREADS), 0, s>>>(w, a, C, sums, m, n, k);

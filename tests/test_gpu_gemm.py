@@ -114,6 +114,25 @@ def test_mul_mat_few_rows(q8, oracle, n, k):
         assert rel_l2(got[0], y0) < 2e-6
 
 
+@pytest.mark.parametrize("m,n,k", [(6, 24577, 256), (33, 24640, 384), (64, 24576 + 96, 128), (40, 30000, 640)])
+def test_few_rows_on_a_wide_matrix(q8, oracle, m, n, k):
+    # >= 192 column blocks of 128 rows: the tile kernel takes the batched-decode shapes too (activation tiles shared through
+    # LDS, weight loads that bypass the caches); ragged N (a last column block with one to three strips, a last strip with
+    # one row), one and two activation strips with padding rows, K sets of one, two and four groups, integer sums and fp32
+    w, x, aq = _inputs(oracle, m, n, k, seed=m + n)
+    wt, aqt = q8.tile(to_dev(w), n, k), q8.tile(to_dev(aq.reshape(-1)), m, k)
+    sums = to_host(q8.debug_block_sums(wt, aqt, m, n, k, path=3))
+    for i in range(m):
+        assert np.array_equal(sums[i], oracle.block_sums_gemv(w, aq[i], n, k)), i
+    got = to_host(q8.gemm(wt, aqt, m, n, k, tiled=True))
+    assert rel_l2(got, oracle.gemm(w, aq, m, n, k)) <= REL_L2_TOL
+    for i in range(m):
+        assert rel_l2(got[i], oracle.gemv(w, aq[i], n, k)) <= REL_L2_TOL, i
+    res = oracle.fill_activations(7, m * n).reshape(m, n)
+    got_r = to_host(q8.gemm_residual(wt, aqt, to_dev(res), m, n, k))
+    assert np.array_equal(got_r, got + res)
+
+
 def test_mul_mat_batch_mixed_rows(q8, oracle):
     # one native call, five projections: two mat-vecs sharing x (one launch), a 3-row op with no workspace use, two 8-row ops sharing the quantized x
     import torch
