@@ -221,7 +221,7 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		*reinterpret_cast<uint32_t*>(lds + ((tid & 255) >> 2) * STAGE_BYTES + DATA_BYTES + 4 * (tid & 3)) = 0u;
 	}
 	// every address below is a wave-uniform part (scalar registers, advanced by scalar adds) plus one of three lane constants
-	const uint32_t lane16 = 16u * lane, lane4 = 4u * lane, sc8 = 8u * (lane & 31);
+	const uint32_t lane16 = 16u * lane;
 	const int64_t w_off	  = uniform_i64(macro_offset(min(ns, n_strips - 1), g_base, groups));
 	struct w_regs {
 		v4i q[GROUP_BLOCKS];
@@ -235,12 +235,12 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	for (int j = 0; j < TM; ++j) {
 		const int u = TM * wave + j;
 		a_off[j]	= uniform_i64(macro_offset(min(ms0 + u / 4, m_strips - 1), g_base, groups) + (u % 4) * TILE_BYTES);
-		a_dst[j]	= (u / 4) * MACRO_BYTES + (u % 4) * TILE_BYTES + lane16;
+		a_dst[j]	= (u / 4) * MACRO_BYTES + (u % 4) * TILE_BYTES; // + 16 * lane at the store
 	}
 	// every wave copies a dword per lane of a scale table (waves >= TM: strip TM-1's again, stored nowhere), so that all waves
 	// issue the same loads
 	const int64_t sc_off  = uniform_i64(macro_offset(min(ms0 + min(wave, TM - 1), m_strips - 1), g_base, groups) + MACRO_D_OFFSET);
-	const uint32_t sc_dst = wave < TM ? wave * MACRO_BYTES + MACRO_D_OFFSET + lane4 : 2 * STAGE_BYTES + lane4;
+	const uint32_t sc_dst = wave < TM ? wave * MACRO_BYTES + MACRO_D_OFFSET : 2 * STAGE_BYTES; // + 4 * lane at the store
 	const uint32_t sc_stage = wave < TM ? STAGE_BYTES : 0; // the spare area is not staged
 	struct a_regs {
 		v4i q[TM];
@@ -248,8 +248,9 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	};
 	auto fetch_a = [&](int g, a_regs& r) {
 		const int64_t adv = static_cast<int64_t>(g) * MACRO_BYTES;
-		uint32_t l16 = lane16, l4 = lane4;
-		asm volatile("" : "+v"(l16), "+v"(l4));
+		uint32_t l16 = lane16;
+		asm volatile("" : "+v"(l16));
+		const uint32_t l4 = l16 >> 2;
 #pragma unroll
 		for (int j = 0; j < TM; ++j) {
 			r.q[j] = load_sv<v4i, false>(scalar_base(A, a_off[j] + adv), l16);
@@ -257,18 +258,21 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		r.d = load_sv<uint32_t, false>(scalar_base(A, sc_off + adv), l4);
 	};
 	auto stash_a = [&](int stage, const a_regs& r) {
-		uint8_t* p = lds + stage * STAGE_BYTES;
+		uint8_t* p	 = lds + stage * STAGE_BYTES;
+		uint32_t l16 = lane16;
+		asm volatile("" : "+v"(l16)); // wave-uniform offsets stay in scalar registers, added here, instead of one more lane constant each
 #pragma unroll
 		for (int j = 0; j < TM; ++j) {
-			*reinterpret_cast<v4i*>(p + a_dst[j]) = r.q[j];
+			*reinterpret_cast<v4i*>(p + a_dst[j] + l16) = r.q[j];
 		}
-		*reinterpret_cast<uint32_t*>(lds + stage * sc_stage + sc_dst) = r.d;
+		*reinterpret_cast<uint32_t*>(lds + stage * sc_stage + sc_dst + (l16 >> 2)) = r.d;
 	};
 	auto fetch_w = [&](int g, w_regs& r) {
 		const int64_t at = w_off + static_cast<int64_t>(g) * MACRO_BYTES;
 		const gptr_u8 p	 = scalar_base(W, at);
-		uint32_t l16 = lane16, l8 = sc8;
-		asm volatile("" : "+v"(l16), "+v"(l8)); // the widening of a lane offset has to stay beside its loads for scalar base + 32-bit lane offset to be picked as the addressing mode
+		uint32_t l16 = lane16;
+		asm volatile("" : "+v"(l16));
+		const uint32_t l8 = (l16 & 0x1F0u) >> 1; // the widening of a lane offset has to stay beside its loads for scalar base + 32-bit lane offset to be picked as the addressing mode
 #pragma unroll
 		for (int k = 0; k < GROUP_BLOCKS; ++k) {
 			r.q[k] = load_sv<v4i, STREAM>(p + k * TILE_BYTES, l16);
@@ -302,36 +306,51 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 			cur.d = v2u{ 0u, 0u };
 		}
 		const uint8_t* stage = lds + (g & 1) * STAGE_BYTES;
+		// the operand of unit u + 1 is read from LDS before unit u's arithmetic starts: one exposed LDS latency per trip, not eight
+		constexpr int UNITS = GROUP_BLOCKS * TM;
+		auto read_a = [&](int u, v4i& a, uint32_t& sc) {
+			const int t = u / TM, i = u % TM;
+			a  = *reinterpret_cast<const v4i*>(stage + i * MACRO_BYTES + t * TILE_BYTES + 16 * lane);
+			sc = *reinterpret_cast<const uint16_t*>(stage + (half ? 0 : i * MACRO_BYTES) + a_sc_rel + 2 * t);
+		};
+		v4i a_cur;
+		uint32_t s_cur;
+		read_a(0, a_cur, s_cur);
 #pragma unroll
-		for (int t = 0; t < GROUP_BLOCKS; ++t) {
+		for (int u = 0; u < UNITS; ++u) {
+			const int t = u / TM, i = u % TM;
+			v4i a_nxt		= a_cur;
+			uint32_t s_nxt	= s_cur;
+			if (u + 1 < UNITS) {
+				read_a(u + 1, a_nxt, s_nxt);
+			}
+			__builtin_amdgcn_sched_barrier(0);
 			const uint32_t wd = (t < 2) ? cur.d.x : cur.d.y;
 			const v2u w_sc	  = v2u{ (t & 1) ? (wd >> 16) : (wd & 0xFFFFu), 0u };
+			const v2u a_sc	  = v2u{ s_cur, 0u };
+			const v16i zi	  = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+			const v16f zf	  = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+			const v16i sv	  = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_cur, cur.q[t], zi, 0, 0, 0);
+			if constexpr (DUMP) {
+				const int n = ns * 32 + (lane & 31);
 #pragma unroll
-			for (int i = 0; i < TM; ++i) {
-				asm volatile("" ::: "memory");
-				const v4i a		= *reinterpret_cast<const v4i*>(stage + i * MACRO_BYTES + t * TILE_BYTES + 16 * lane);
-				const v2u a_sc	= v2u{ *reinterpret_cast<const uint16_t*>(stage + (half ? 0 : i * MACRO_BYTES) + a_sc_rel + 2 * t), 0u };
-				const v16i zi	= { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-				const v16f zf	= { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-				const v16i sv	= __builtin_amdgcn_mfma_i32_32x32x32_i8(a, cur.q[t], zi, 0, 0, 0);
-				if constexpr (DUMP) {
-					const int n = ns * 32 + (lane & 31);
-#pragma unroll
-					for (int e = 0; e < 16; ++e) {
-						const int m = (ms0 + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-						if (m < M && n < N) {
-							sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + (g_base + g) * GROUP_BLOCKS + t] = sv[e];
-						}
+				for (int e = 0; e < 16; ++e) {
+					const int m = (ms0 + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+					if (m < M && n < N) {
+						sums[(static_cast<int64_t>(m) * N + n) * (groups * GROUP_BLOCKS) + (g_base + g) * GROUP_BLOCKS + t] = sv[e];
 					}
-				} else {
-					const v16f pv = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, a_sc), __builtin_bit_cast(v4h, w_sc), zf, 0, 0, 0);
-#pragma unroll
-					for (int e = 0; e < 16; ++e) {
-						acc[i][e] = fmaf(static_cast<float>(sv[e]), pv[e], acc[i][e]);
-					}
-					asm volatile("" : "+v"(acc[i]));
 				}
+			} else {
+				const v16f pv = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, a_sc), __builtin_bit_cast(v4h, w_sc), zf, 0, 0, 0);
+#pragma unroll
+				for (int e = 0; e < 16; ++e) {
+					acc[i][e] = fmaf(static_cast<float>(sv[e]), pv[e], acc[i][e]);
+				}
+				asm volatile("" : "+v"(acc[i]));
 			}
+			__builtin_amdgcn_sched_barrier(0);
+			a_cur = a_nxt;
+			s_cur = s_nxt;
 		}
 		stash_a((g + 1) & 1, pre);
 		__syncthreads();
