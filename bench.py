@@ -275,12 +275,35 @@ def main() -> int:
         torch.cuda.empty_cache()
     if not args.no_decode:
         result["decode"] = decode_step(args.decode_tokens)
+        torch.cuda.empty_cache()
+        surface = dispatch_surface()
+        if surface is not None:
+            result["dispatch_surface"] = surface
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
 
     print(json.dumps(result))
     return 0
+
+
+def dispatch_surface() -> dict | None:
+    """The decode token and the FFN step once more, this time entered the way the reference's scheduler enters them: through
+    kernel_dispatcher<config, eval_time, core>::impl of the C++ dispatch header (tests/cpp/time_mega_dispatch.cpp, a host program
+    built beside the host tests and run here as a child process; it links the library only).  None when it has not been built."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "cpp", "time_mega_dispatch")
+    if not os.path.exists(exe):
+        return None
+    try:
+        res = subprocess.run([exe, "30", "3"], capture_output=True, text=True, timeout=180)
+        line = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+        if res.returncode != 0 or not line:
+            return {"error": (res.stdout + res.stderr)[-400:], "returncode": res.returncode}
+        return json.loads(line[-1])
+    except (subprocess.TimeoutExpired, OSError, ValueError) as e:
+        return {"error": repr(e)[:400]}
 
 
 def gemv_shapes(steps: int) -> dict:
@@ -383,7 +406,22 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
 
         wall, ksec, n = timed(0, fn, 1)
         ach = nbytes / ksec / 1e9
+        # the two fused forms of the prefill path, same shape: RMS norm . weight -> quantize, SiLU(gate) . up -> quantize
+        nw = q8_0.fill_activations(5, K)
+        up = q8_0.fill_activations(6, M * K).reshape(M, K)
+
+        def fn_norm():
+            _lib.check("nh_q8_0_rms_norm_quantize_tiled", lib.nh_q8_0_rms_norm_quantize_tiled(x.data_ptr(), nw.data_ptr(), C.c_float(1e-5), out.data_ptr(), M, K, stream))
+
+        def fn_silu():
+            _lib.check("nh_q8_0_silu_mul_quantize_tiled", lib.nh_q8_0_silu_mul_quantize_tiled(x.data_ptr(), up.data_ptr(), out.data_ptr(), M, K, stream))
+
+        fused = []
+        for entry, f, b in (("nh_q8_0_rms_norm_quantize_tiled", fn_norm, nbytes + 4 * K), ("nh_q8_0_silu_mul_quantize_tiled", fn_silu, nbytes + 4 * M * K)):
+            _, ks, _ = timed(0, f, 1)
+            fused.append({"entry": entry, "avg_launch_us": round(ks * 1e6, 3), "bytes_per_launch": b, "GBs": round(b / ks / 1e9, 1)})
         return {
+            "fused_forms": fused,
             "metric": "Q8_0 activation quantize GB/s", "value": round(nbytes / wall / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
             "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "dtype": "fp32 -> int8 + fp16 scale", "data": "synthetic",
             "config": {"workload": f"activation quantize, fp32 [{M}x{K}] -> tiled Q8_0 (cache-resident at this size: 10.6 MB)"},

@@ -15,9 +15,10 @@ HOST_TEST_SRC = os.path.join(HERE, "test_mul_mat_dispatch.cpp")
 HOST_TEST_BIN = os.path.join(HERE, "test_mul_mat_dispatch")
 MEGA_TEST_BIN = os.path.join(HERE, "test_mega_dispatch")  # the live dispatch point (core_types key), run on the GPU
 REFERENCE_MODE_BIN = os.path.join(HERE, "test_reference_mode_compiles")  # the headers against the reference's own primary template
+TIME_MEGA_BIN = os.path.join(HERE, "time_mega_dispatch")  # decode token timed through the dispatch point (links the library only, not the checker)
 
 
-def _build_one(src: str, out: str) -> str:
+def _build_one(src: str, out: str, with_checker: bool = True) -> str:
     from nihilus_amd.build import PKG_DIR, hipcc
 
     cxx = os.path.join(os.path.dirname(hipcc()), "amdclang++")
@@ -26,9 +27,10 @@ def _build_one(src: str, out: str) -> str:
     oracle_dir = os.path.join(ROOT, "oracle")
     cmd = [
         cxx, "-std=c++23", "-O2", "-Wall", "-Wextra", "-I", os.path.join(ROOT, "include"), os.path.join(HERE, src), "-o", out,
-        "-L", PKG_DIR, "-lnihilus_q8_hip", "-L", oracle_dir, "-lq8_0_oracle",
-        "-Wl,-rpath,$ORIGIN/../../nihilus_amd", "-Wl,-rpath,$ORIGIN/../../oracle", "-Wl,-rpath,/opt/rocm/lib",
+        "-L", PKG_DIR, "-lnihilus_q8_hip", "-Wl,-rpath,$ORIGIN/../../nihilus_amd", "-Wl,-rpath,/opt/rocm/lib",
     ]
+    if with_checker:
+        cmd += ["-L", oracle_dir, "-lq8_0_oracle", "-Wl,-rpath,$ORIGIN/../../oracle"]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"host test build failed:\n{' '.join(cmd)}\n{res.stderr}")
@@ -37,6 +39,7 @@ def _build_one(src: str, out: str) -> str:
 
 def build_host_tests() -> str:
     _build_one("test_mega_dispatch.cpp", MEGA_TEST_BIN)
+    _build_one("time_mega_dispatch.cpp", TIME_MEGA_BIN, with_checker=False)
     _build_one("test_reference_mode_compiles.cpp", REFERENCE_MODE_BIN)
     return _build_one("test_mul_mat_dispatch.cpp", HOST_TEST_BIN)
 

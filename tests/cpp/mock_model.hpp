@@ -24,13 +24,30 @@ namespace nihilus {
 		static constexpr uint64_t n_embd_kv_gqa{ rope_dimension_count * attention_head_count_kv };
 	};
 
+	// the shapes of the decode benchmark configuration (LLaMA-3-8B)
+	struct llama3_8b_traits {
+		static constexpr float layer_norm_rms_epsilon{ 1e-5f };
+		static constexpr uint32_t vocab_size{ 128256 };
+		static constexpr uint32_t embedding_length{ 4096 };
+		static constexpr uint32_t block_count{ 32 };
+		static constexpr uint32_t feed_forward_length{ 14336 };
+		static constexpr uint32_t attention_head_count{ 32 };
+		static constexpr uint32_t attention_head_count_kv{ 8 };
+		static constexpr uint32_t rope_dimension_count{ embedding_length / attention_head_count };
+		static constexpr uint64_t n_embd_kv_gqa{ rope_dimension_count * attention_head_count_kv };
+	};
+
+#ifndef NH_MOCK_MODEL_TRAITS
+	#define NH_MOCK_MODEL_TRAITS tiny_llama_traits // a translation unit that wants the other set defines this before the include
+#endif
+
 	struct mock_config {
 		static constexpr device_types device_type{ device_types::gpu };
 		static constexpr kernel_type_profiles kernel_type_profile{ kernel_type_profiles::q8_gqa };
 		static constexpr bool exceptions{ true };
 		static constexpr bool dev{ false };
 		static constexpr uint64_t max_sequence_length{ 64 };
-		using model_traits_type = tiny_llama_traits;
+		using model_traits_type = NH_MOCK_MODEL_TRAITS;
 	};
 
 	// one graph node: raw storage (global or per block) + the runtime sequence length + its enumerator
@@ -99,7 +116,7 @@ namespace nihilus {
 	template<> struct core_traits_old<mock_config, core_types::mega_qkv_prep_and_cache_publish> {
 		static constexpr core_types core_type{ core_types::mega_qkv_prep_and_cache_publish };
 		using config_type = mock_config;
-		using mtt		  = tiny_llama_traits;
+		using mtt		  = NH_MOCK_MODEL_TRAITS;
 		mock_ops<mock_op<mega_qkv_prep_and_cache_publish_types::q_out, data_strategy_types::global>> values{};
 		struct kernel_data_ptrs_type {
 			NH_MOCK_GETTER(inp_embd_data, const)
@@ -136,7 +153,7 @@ namespace nihilus {
 	template<> struct core_traits_old<mock_config, core_types::mega_attention_apply> {
 		static constexpr core_types core_type{ core_types::mega_attention_apply };
 		using config_type = mock_config;
-		using mtt		  = tiny_llama_traits;
+		using mtt		  = NH_MOCK_MODEL_TRAITS;
 		mock_ops<mock_op<mega_attention_apply_types::ffn_inp, data_strategy_types::global>> values{};
 		struct kernel_data_ptrs {
 			NH_MOCK_GETTER(q_input_data, const)
@@ -167,7 +184,7 @@ namespace nihilus {
 	template<> struct core_traits_old<mock_config, core_types::mega_ffn> {
 		static constexpr core_types core_type{ core_types::mega_ffn };
 		using config_type = mock_config;
-		using mtt		  = tiny_llama_traits;
+		using mtt		  = NH_MOCK_MODEL_TRAITS;
 		mock_ops<mock_op<mega_ffn_types::l_out, data_strategy_types::global>> values{};
 		struct kernel_data_ptrs {
 			NH_MOCK_GETTER(ffn_inp_data, const)
@@ -196,7 +213,7 @@ namespace nihilus {
 	template<> struct core_traits_old<mock_config, core_types::final_norm_and_sampling> {
 		static constexpr core_types core_type{ core_types::final_norm_and_sampling };
 		using config_type = mock_config;
-		using mtt		  = tiny_llama_traits;
+		using mtt		  = NH_MOCK_MODEL_TRAITS;
 		mock_ops<mock_op<final_norm_and_sampling_types::result_token_id, data_strategy_types::global>> values{};
 		struct kernel_data_ptrs {
 			NH_MOCK_GETTER(l_out_data, const)

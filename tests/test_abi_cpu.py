@@ -154,7 +154,7 @@ def test_cpp_live_dispatch_point_compiles_against_the_reference_declaration():
     # test-local header whose primary template is the reference's own declaration of the live specialisation point; all eight
     # specialisations are instantiated through the reference's caller-side template.  Also the stand-alone build's static checks.
     b = _host_tests()
-    if not (os.path.exists(b.REFERENCE_MODE_BIN) and os.path.exists(b.MEGA_TEST_BIN)):
+    if not (os.path.exists(b.REFERENCE_MODE_BIN) and os.path.exists(b.MEGA_TEST_BIN) and os.path.exists(b.TIME_MEGA_BIN)):
         import oracle  # noqa: F401
 
         b.build_host_tests()
@@ -174,6 +174,19 @@ def test_cpp_live_dispatch_point_on_gpu():
     res = subprocess.run([b.MEGA_TEST_BIN], capture_output=True, text=True, timeout=120)
     assert res.returncode == 0, res.stdout + res.stderr
     assert "mega dispatch ok" in res.stdout
+
+
+@pytest.mark.gpu
+def test_decode_token_timed_through_the_dispatch_point():
+    # the measurement's own entry through the C++ dispatch header: a whole LLaMA-3-8B-shaped token and the FFN core alone
+    import json
+
+    b = _host_tests()
+    res = subprocess.run([b.TIME_MEGA_BIN, "3", "1"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout + res.stderr
+    out = json.loads(res.stdout.strip().splitlines()[-1])
+    assert out["decode"]["weight_bytes_per_token"] == 7973699584 and out["decode"]["tok_s"] > 100
+    assert out["mega_ffn"]["GBs"] > 1000
 
 
 @pytest.mark.gpu
