@@ -279,6 +279,15 @@ def main() -> int:
         surface = dispatch_surface()
         if surface is not None:
             result["dispatch_surface"] = surface
+        floor = launch_floor()
+        if floor is not None:
+            # what the ordered token's launches cost before they move a byte, and the token time that this and the peak bandwidth leave
+            d = result["decode"]
+            per = floor.get("one_load_kernel_queued_us", [0.0])[0]
+            if per > 0:
+                floor["decode_lower_bound_ms"] = round((d["launches_per_token"] * per + d["weight_bytes_per_token"] / (HBM_PEAK_GBS * 1e3)) * 1e-3, 4)
+                floor["decode_upper_bound_tok_s"] = round(1e3 / floor["decode_lower_bound_ms"], 1)
+            result["launch_floor"] = floor
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
@@ -298,6 +307,24 @@ def dispatch_surface() -> dict | None:
         return None
     try:
         res = subprocess.run([exe, "30", "3"], capture_output=True, text=True, timeout=180)
+        line = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+        if res.returncode != 0 or not line:
+            return {"error": (res.stdout + res.stderr)[-400:], "returncode": res.returncode}
+        return json.loads(line[-1])
+    except (subprocess.TimeoutExpired, OSError, ValueError) as e:
+        return {"error": repr(e)[:400]}
+
+
+def launch_floor() -> dict | None:
+    """Device-side cost of a dispatch that does nothing (tests/cpp/launch_floor_probe.hip, a HIP program of its own run as a child
+    process): an empty kernel and a one-load kernel, queued behind a kernel that holds the device.  None when it has not been built."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "cpp", "launch_floor_probe")
+    if not os.path.exists(exe):
+        return None
+    try:
+        res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
         line = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
         if res.returncode != 0 or not line:
             return {"error": (res.stdout + res.stderr)[-400:], "returncode": res.returncode}

@@ -154,7 +154,7 @@ def test_cpp_live_dispatch_point_compiles_against_the_reference_declaration():
     # test-local header whose primary template is the reference's own declaration of the live specialisation point; all eight
     # specialisations are instantiated through the reference's caller-side template.  Also the stand-alone build's static checks.
     b = _host_tests()
-    if not (os.path.exists(b.REFERENCE_MODE_BIN) and os.path.exists(b.MEGA_TEST_BIN) and os.path.exists(b.TIME_MEGA_BIN)):
+    if not (os.path.exists(b.REFERENCE_MODE_BIN) and os.path.exists(b.MEGA_TEST_BIN) and os.path.exists(b.TIME_MEGA_BIN) and os.path.exists(b.LAUNCH_FLOOR_BIN)):
         import oracle  # noqa: F401
 
         b.build_host_tests()
@@ -174,6 +174,17 @@ def test_cpp_live_dispatch_point_on_gpu():
     res = subprocess.run([b.MEGA_TEST_BIN], capture_output=True, text=True, timeout=120)
     assert res.returncode == 0, res.stdout + res.stderr
     assert "mega dispatch ok" in res.stdout
+
+
+@pytest.mark.gpu
+def test_launch_floor_probe_runs():
+    import json
+
+    b = _host_tests()
+    res = subprocess.run([b.LAUNCH_FLOOR_BIN], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout + res.stderr
+    out = json.loads(res.stdout.strip().splitlines()[-1])
+    assert all(0.2 < v < 20.0 for v in out["empty_kernel_queued_us"] + out["one_load_kernel_queued_us"])
 
 
 @pytest.mark.gpu
