@@ -12,7 +12,8 @@
  * the reference has no FFI for this path; its boundary is the class-template specialisation point
  * kernel_dispatcher_impl<config, core_traits, device, arch, ...>::impl (common/kernel_traits.hpp:382-383,
  * called from infra/monolithic_dispatcher.hpp:41-63).  The C++ header mul_mat_dispatch.hpp supplies
- * those specialisations for device_types::gpu and forwards to the functions below.
+ * those specialisations for device_types::gpu and forwards to the functions below; mega_dispatch.hpp does the same
+ * for the reference's live dispatch point (the core_types key).
  *
  * Streams
  *   Launches that hand data between workgroups do so through scratch memory that the library keeps per GPU (made on first
@@ -22,6 +23,8 @@
  *   the other stream drain first.  A call that would use the scratch while a launch from a different stream may still be
  *   running returns NH_ERR_BUSY and launches nothing (not detected: work on a capturing stream, work that followed a
  *   launch on the NULL stream, and replays of captured graphs, which the caller must keep from overlapping).
+ *   The check queries the other stream; it does so in the relaxed capture mode, so it may run while a third stream of the
+ *   calling thread is being captured in the global mode without disturbing that capture.
  *   A kernel that waits for another workgroup's data does so for a bounded time; if it gives up, the output holds NaN and
  *   the next nh_stream_sync (or nh_q8_0_last_error) on that GPU returns NH_ERR_DEVICE_TIMEOUT once.
  *

@@ -214,6 +214,20 @@ inline bool stream_is_capturing(hipStream_t s) {
 	return st != hipStreamCaptureStatusNone;
 }
 
+// hipStreamQuery of a stream that is not itself capturing, safe to call while ANOTHER stream of this thread is being captured
+// in the global mode (where a query would be refused and would invalidate that capture): the thread's capture mode is
+// relaxed for the duration of the call.
+inline hipError_t query_stream_any_capture_mode(hipStream_t s) {
+	hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+	if (hipThreadExchangeStreamCaptureMode(&mode) != hipSuccess) {
+		(void)hipGetLastError();
+		return hipStreamQuery(s);
+	}
+	const hipError_t q = hipStreamQuery(s);
+	(void)hipThreadExchangeStreamCaptureMode(&mode);
+	return q;
+}
+
 // When timing is on for `kind` and the event pool has room, hands out an event pair for the next launch.
 bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop);
 

@@ -294,7 +294,7 @@ static hipError_t get_skinny_scratch(skinny_scratch* out, bool launching = false
 	}
 	if (launching && !stream_is_capturing(s)) {
 		if (sc.has_user && sc.user != s && sc.user != nullptr && !stream_is_capturing(sc.user)) {
-			const hipError_t q = hipStreamQuery(sc.user);
+			const hipError_t q = query_stream_any_capture_mode(sc.user);
 			if (q == hipErrorNotReady) {
 				return q;
 			}

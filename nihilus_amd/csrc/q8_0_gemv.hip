@@ -207,7 +207,7 @@ namespace {
 		if (stream_is_capturing(prev)) {
 			return hipSuccess; // must not be queried; its launches take forms that keep no state in the scratch
 		}
-		const hipError_t q = hipStreamQuery(prev);
+		const hipError_t q = query_stream_any_capture_mode(prev);
 		if (q == hipErrorNotReady) {
 			return q;
 		}

@@ -106,3 +106,37 @@ def test_captured_batch_of_independent_mat_vecs(q8, oracle):
             assert rel_l2(got[i], to_host(ys[i])) < 2e-6, (seed, i)
     aq = oracle.quantize_rows(to_host(xs[2]).reshape(1, -1))[0]
     assert rel_l2(got[2], oracle.gemv(to_host(q8.untile(ws[2], *shapes[2])), aq, *shapes[2])) <= REL_L2_TOL
+
+
+def test_eager_split_launch_on_another_stream_while_a_stream_captures(q8, oracle):
+    # Global-mode capture (torch's default) refuses stream queries from the capturing thread and a refused call invalidates the
+    # capture.  The scratch's one-stream guard queries the stream of the previous K-split launch: it has to do so without
+    # disturbing a capture that is going on elsewhere in the thread.
+    import torch
+
+    from nihilus_amd import _lib
+
+    lib = _lib.lib()
+    _lib.check("nh_q8_0_prepare", lib.nh_q8_0_prepare())
+    n, k = 1024, 14336  # K split over workgroups when launched eagerly
+    w = oracle.fill_weights(21, n, k)
+    x = oracle.fill_activations(21, k)
+    wt, xd = q8.tile(to_dev(w), n, k), to_dev(x)
+    y_c = torch.empty(n, dtype=torch.float32, device="cuda")
+    y_b = torch.empty(n, dtype=torch.float32, device="cuda")
+    y_g = torch.empty(n, dtype=torch.float32, device="cuda")
+    b, c = torch.cuda.Stream(), torch.cuda.Stream()
+    assert lib.nh_q8_0_gemv_tiled_f32(wt.data_ptr(), xd.data_ptr(), y_c.data_ptr(), n, k, c.cuda_stream) == 0  # the scratch's user is now stream c
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cap = torch.cuda.current_stream().cuda_stream
+        assert lib.nh_q8_0_gemv_tiled_f32(wt.data_ptr(), xd.data_ptr(), y_g.data_ptr(), n, k, cap) == 0  # captured: the unsplit form
+        # eager, on stream b, in the middle of the capture: the guard looks at stream c
+        assert lib.nh_q8_0_gemv_tiled_f32(wt.data_ptr(), xd.data_ptr(), y_b.data_ptr(), n, k, b.cuda_stream) == 0
+    b.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    want = oracle.gemv(w, oracle.quantize_rows(x)[0], n, k)
+    assert rel_l2(to_host(y_b), want) <= REL_L2_TOL and np.array_equal(to_host(y_b), to_host(y_c))
+    assert rel_l2(to_host(y_g), want) <= REL_L2_TOL
