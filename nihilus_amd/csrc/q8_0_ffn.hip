@@ -45,6 +45,7 @@ struct ffn_args {
 	int split_shift; // a consumer strip's K range goes over (1 << split_shift) workgroups of 16 waves
 	unsigned* error_word; // device-visible host word: set when a consumer gives up waiting for a producer
 	int spin_limit; // polls before it does
+	uint64_t* x_words; // scratch (NORM): the normalised, quantized input row, published by the first producer workgroup for the others; null: each works it out
 };
 
 template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
@@ -62,12 +63,6 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 		__shared__ __align__(16) float act_f[STRIP_ROWS];
 		__shared__ float norm_red[16];
 		__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1];
-		gemv_norm norm_state;
-		gemv_norm* norm = nullptr;
-		if constexpr (NORM) { // the row's scale first
-			gemv_norm_begin(norm_state, a.x, a.norm_w, xs_w[NORM ? wave : 0], norm_red, a.norm_eps, a.groups_p * GROUP_K, lane, wave);
-			norm = &norm_state;
-		}
 		const int matrix	   = wave >> 3;
 		const int slot		   = wave & 7;
 		const int strip		   = wg;
@@ -76,11 +71,36 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 		const uint8_t* w_strip = (matrix ? a.w_up : a.w_gate) + macro_offset(strip, 0, a.groups_p);
 		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
 		float acc			   = 0.0f;
-		if constexpr (!LOOP) {
-			acc = gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, 0, norm);
+		auto walk = [&]<int XMODE, bool WITH_NORM>(const void* x_from, void* dump_to, gemv_norm* norm) {
+			if constexpr (!LOOP) {
+				return gemv_chunk<TILES, XMODE, DUMP_NONE, WITH_NORM>(w_strip, x_from, dump_to, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, a.epoch, norm, 0, a.spin_limit);
+			} else {
+				float sum = 0.0f;
+				for (int gc = g0; gc < g1; gc += TILES) {
+					sum += gemv_chunk<TILES, XMODE, DUMP_NONE, WITH_NORM>(w_strip, x_from, dump_to, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false, a.epoch, norm, 0,
+						a.spin_limit);
+					__builtin_amdgcn_wave_barrier();
+				}
+				return sum;
+			}
+		};
+		if constexpr (NORM) {
+			// one row, one norm: the first producer workgroup works the normalised, quantized row out (its gate waves cover all of K
+			// between them and publish what they stage), the others read it from there
+			if (!a.x_words || wg == 0) {
+				gemv_norm norm_state; // the row's scale first (a workgroup barrier inside)
+				gemv_norm_begin(norm_state, a.x, a.norm_w, xs_w[NORM ? wave : 0], norm_red, a.norm_eps, a.groups_p * GROUP_K, lane, wave);
+				norm_state.publish = matrix == 0 ? a.x_words : nullptr;
+				norm_state.epoch   = a.epoch;
+				acc				   = walk.template operator()<X_F32, true>(a.x, nullptr, &norm_state);
+			} else {
+				acc = walk.template operator()<X_PUBLISHED_EARLY, false>(a.x_words, a.error_word, nullptr);
+			}
+		} else if constexpr (!LOOP) {
+			acc = gemv_chunk<TILES, X_F32, DUMP_NONE, false>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, 0, nullptr);
 		} else {
 			for (int gc = g0; gc < g1; gc += TILES) {
-				acc += gemv_chunk<TILES, X_F32, DUMP_NONE, NORM>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false, 0, norm);
+				acc += gemv_chunk<TILES, X_F32, DUMP_NONE, false>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), a.groups_p, lane, row_l, a.n_ff, false, 0, nullptr);
 				__builtin_amdgcn_wave_barrier();
 			}
 		}
@@ -235,6 +255,7 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	a.groups_p	 = static_cast<int>(K / GROUP_K);
 	a.groups_c	 = groups_c;
 	a.producers	 = static_cast<int>(n_ff / STRIP_ROWS);
+	a.x_words	 = norm_w && a.producers >= FFN_SHARED_X_MIN_PRODUCERS && K <= GEMV_SHARED_X_MAX_K ? sc.x_words : nullptr;
 	a.p_per_slot = a.groups_p / (GEMV_WAVES / 2);
 	a.p_rem		 = a.groups_p % (GEMV_WAVES / 2);
 	int shift	 = 0;

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_blocks_kernel(const uint8_t* 
 //     matrix with few rows reaches every CU without partial sums.
 template<int TILES, bool XF32, int DUMP, bool LOOP, bool NORM, int RS = 1>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segments seg, const void* __restrict__ xin, void* __restrict__ dump, uint64_t* __restrict__ tagged,
-	unsigned epoch, int groups, int split_shift, const float* __restrict__ norm_w, float norm_eps) {
+	unsigned epoch, int groups, int split_shift, const float* __restrict__ norm_w, float norm_eps, uint64_t* __restrict__ x_words, unsigned* error_word, int spin_limit) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K]; // each wave's activation quants, block jj at 32*jj
 	__shared__ float norm_red[16];
 	__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1]; // each wave's slice of the norm weights
@@ -140,19 +140,42 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 	const uint8_t* w_strip = DUMP == DUMP_X ? nullptr : seg.W[sidx] + macro_offset(strip, 0, groups);
 	const int row_l		   = strip * STRIP_ROWS + (lane & 31);
 	float acc			   = 0.0f;
-	gemv_norm norm_state;
-	gemv_norm* norm = nullptr;
-	if constexpr (NORM) { // RMS norm * weight in front of the quantizer: the row's scale first
-		gemv_norm_begin(norm_state, static_cast<const float*>(xin), norm_w, xs_w[NORM ? wave : 0], norm_red, norm_eps, groups * GROUP_K, lane, wave);
-		norm = &norm_state;
-	}
-	if constexpr (!LOOP) {
-		// the host picked splits so that g1 - g0 <= TILES: straight-line code, every load of the wave in flight at once
-		acc = gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, 0, norm, rowpart);
+	// the wave's K range, in one piece when the host picked splits so that g1 - g0 <= TILES (straight-line code, every load of the
+	// wave in flight at once), else walked in chunks of TILES groups (K too long for that within the host's scratch limits)
+	auto walk = [&]<int XMODE, bool WITH_NORM>(const void* x_from, void* dump_to, gemv_norm* norm) {
+		if constexpr (!LOOP) {
+			return gemv_chunk<TILES, XMODE, DUMP, WITH_NORM, RS>(w_strip, x_from, dump_to, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, epoch, norm, rowpart, spin_limit);
+		} else {
+			float sum = 0.0f;
+			for (int gc = g0; gc < g1; gc += TILES) {
+				sum += gemv_chunk<TILES, XMODE, DUMP, WITH_NORM, RS>(w_strip, x_from, dump_to, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, epoch, norm, rowpart, spin_limit);
+				__builtin_amdgcn_wave_barrier(); // the next chunk overwrites this wave's LDS slice
+			}
+			return sum;
+		}
+	};
+	if constexpr (NORM) {
+		// RMS norm * weight in front of the quantizer.  With x_words the row is normalised and quantized once per launch: by the
+		// workgroups of the first strip (one per K split, each on its K range; the first workgroup alone when strips are cut by
+		// rows), which publish what they stage; everybody else reads it from there.
+		bool works_it_out = true;
+		if constexpr (DUMP == DUMP_NONE) { // (the inspection variants never share)
+			works_it_out = !x_words || (RS > 1 ? blockIdx.x == 0 : gstrip == 0);
+		}
+		if (works_it_out) {
+			gemv_norm norm_state; // the row's scale first (a workgroup barrier inside)
+			gemv_norm_begin(norm_state, static_cast<const float*>(xin), norm_w, xs_w[NORM ? wave : 0], norm_red, norm_eps, groups * GROUP_K, lane, wave);
+			norm_state.publish = x_words;
+			norm_state.epoch   = epoch;
+			acc				   = walk.template operator()<XF32 ? X_F32 : X_BLOCKS, true>(xin, dump, &norm_state);
+		} else if constexpr (DUMP == DUMP_NONE) {
+			acc = walk.template operator()<X_PUBLISHED_EARLY, false>(x_words, error_word, nullptr);
+		}
+	} else if constexpr (!LOOP) {
+		acc = gemv_chunk<TILES, XF32, DUMP, false, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, 0, nullptr, rowpart);
 	} else {
-		// K too long for that within the host's scratch limits: walk the range in chunks of TILES groups
 		for (int gc = g0; gc < g1; gc += TILES) {
-			acc += gemv_chunk<TILES, XF32, DUMP, NORM, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, 0, norm, rowpart);
+			acc += gemv_chunk<TILES, XF32, DUMP, false, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], gc, min(TILES, g1 - gc), groups, lane, row_l, N, gstrip == 0, 0, nullptr, rowpart);
 			__builtin_amdgcn_wave_barrier(); // the next chunk overwrites this wave's LDS slice
 		}
 	}
@@ -232,7 +255,9 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch, hipStream_t s) {
 	gemv_scratch& sc  = st.sc;
 	if (!sc.tagged) {
 		void* p			   = nullptr;
-		const size_t bytes = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS * 8 + (FFN_MAX_HIDDEN / QK) * BLOCK_BYTES;
+		const size_t blocks_end = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS * 8 + (FFN_MAX_HIDDEN / QK) * BLOCK_BYTES;
+		const size_t x_words_at = (blocks_end + 255) / 256 * 256;
+		const size_t bytes		= x_words_at + static_cast<size_t>(GEMV_SHARED_X_MAX_K / QK) * PUBLISHED_WORDS * 8;
 		e				   = hipMalloc(&p, bytes);
 		if (e != hipSuccess) {
 			return e;
@@ -251,6 +276,7 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch, hipStream_t s) {
 		sc.gate_up	  = reinterpret_cast<float*>(sc.tagged + static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS);
 		sc.act_words  = reinterpret_cast<uint64_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
 		sc.act_blocks = reinterpret_cast<uint8_t*>(sc.act_words + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS); // 16-byte aligned: every part before it is a multiple of 16 bytes
+		sc.x_words	  = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(p) + x_words_at);
 		sc.error_word = static_cast<unsigned*>(word);
 	}
 	if (next_epoch) {
@@ -364,24 +390,33 @@ bool gemv_noalloc_fits(int64_t N, int64_t K) {
 	return p.splits == 1 || static_cast<int64_t>(p.strips) * p.splits <= NOALLOC_MAX_SPLIT_UNITS;
 }
 
+// whether a launch with a norm has its first strip's workgroups work the row out for the others (rs: row parts per strip)
+static bool gemv_shares_x(const gemv_plan& p, int rs) {
+	return static_cast<int64_t>(p.strips) * p.splits * rs >= GEMV_SHARED_X_MIN_WORKGROUPS && static_cast<int64_t>(p.groups) * GROUP_K <= GEMV_SHARED_X_MAX_K;
+}
+
 template<int TILES, bool XF32, bool LOOP, bool NORM, int RS = 1> static hipError_t launch_gemv_tiled_n(const gemv_plan& p, const gemv_segments& seg, const void* x, void* dump, int dump_mode, const gemv_scratch& sc, const float* norm_w, float norm_eps, hipStream_t s) {
 	const dim3 grid(static_cast<unsigned>(p.strips * p.splits * RS)), block(GEMV_WAVES * 64);
+	// a norm in a launch of more than one strip, with a fresh epoch in hand: the first strip's workgroups work the row out for all
+	uint64_t* shared_x = NORM && sc.epoch != 0 && gemv_shares_x(p, RS) ? sc.x_words : nullptr;
 	if constexpr (RS > 1) { // row split (unsplit K, production only): RS workgroups per strip, nothing handed over
-		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM, RS>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, 0, norm_w, norm_eps);
+		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM, RS>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, 0, norm_w, norm_eps, shared_x, sc.error_word,
+			sc.spin_limit);
 	} else {
 		int shift = 0;
 		while ((1 << shift) < p.splits) {
 			++shift;
 		}
 		if (dump_mode == DUMP_SUMS) {
-			gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps);
+			gemv_tiled_kernel<TILES, XF32, DUMP_SUMS, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps, nullptr, nullptr, 0);
 			return hipGetLastError();
 		}
 		if (dump_mode == DUMP_X) {
-			gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps);
+			gemv_tiled_kernel<TILES, XF32, DUMP_X, LOOP, NORM><<<grid, block, 0, s>>>(seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps, nullptr, nullptr, 0);
 			return hipGetLastError();
 		}
-		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps);
+		return launch_kernel(KIND_GEMV, gemv_tiled_kernel<TILES, XF32, DUMP_NONE, LOOP, NORM>, grid, block, 0, s, seg, x, dump, sc.tagged, sc.epoch, p.groups, shift, norm_w, norm_eps, shared_x, sc.error_word,
+			sc.spin_limit);
 	}
 }
 
@@ -429,6 +464,14 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 		p.tiles	 = (p.groups + GEMV_WAVES - 1) / GEMV_WAVES;
 	}
 	gemv_scratch sc;
+	if (p.splits == 1 && norm_w && x_is_f32 && dump_mode == DUMP_NONE && !noalloc && gemv_shares_x(p, 1) && !stream_is_capturing(s)) {
+		// the normalised, quantized row goes from the first strip's workgroups to the others through the scratch, tagged with a
+		// fresh epoch; not under capture, where a replay could not renew the epoch: there every workgroup works the row out
+		const hipError_t e = get_gemv_scratch(&sc, true, s);
+		if (e != hipSuccess) {
+			return e;
+		}
+	}
 	if (p.splits > 1) {
 		if (noalloc && p.strips * p.splits > NOALLOC_MAX_SPLIT_UNITS) {
 			return hipErrorInvalidValue; // the caller checks gemv_noalloc_fits first

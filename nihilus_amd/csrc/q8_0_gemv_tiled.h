@@ -30,7 +30,9 @@ enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
 //               wait is bounded: after `spin_limit` polls the wave gives up, returns NaN and stores a non-zero code
 //               in the device-visible error word that `dump` names in this mode (host memory that the next
 //               nh_stream_sync / nh_q8_0_last_error reads), so the kernel always drains and the failure reaches the host.
-enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2 };
+//   X_PUBLISHED_EARLY  the same, with a first read of the words ahead of the weight loads: for slices that are usually there
+//               already when the workgroup starts (a launch's input row, published by its first workgroups).
+enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2, X_PUBLISHED_EARLY = 3 };
 constexpr int PUBLISHED_SPIN_LIMIT = 1 << 20;
 constexpr int PUBLISHED_WORDS	   = 9; // per block: quant dwords 0..7, then the scale
 // codes a kernel leaves in the device-visible error word (nh_q8_0_last_error reports them as NH_ERR_DEVICE_TIMEOUT)
@@ -45,16 +47,24 @@ enum device_error : unsigned { DEVICE_ERROR_NONE = 0, DEVICE_ERROR_PUBLISH_TIMEO
 // Loads return in issue order, so what the staging needs (the slice and its norm weights) is requested BEFORE the weight
 // stream: a load issued after it would only come back behind it.  The norm weights go from memory straight into LDS (no
 // destination registers: the kernel stays at two workgroups per CU).
+// One row, one norm: in a launch of many workgroups only those of the first strip do this (`publish` below); as they stage their
+// slices they also write them out as tagged words, and every other workgroup takes its slice from there (X_PUBLISHED_EARLY)
+// instead of reading the row, the norm weights and working the same blocks out again -- which, norm weights and all, cost the
+// one-launch FFN 3 us of its 34.
 struct gemv_norm {
 	const float* w; // norm weight, fp32 [K]
 	float4* xs_w; // this wave's LDS slice for the norm weights of its activation slice (TILES * 32 float4)
 	float scale; // the row's 1 / rms
+	uint64_t* publish; // non-null: where the staged blocks also go, PUBLISHED_WORDS {epoch, payload} words per block, indexed by block of the row
+	unsigned epoch;
 };
 // red: 16 floats of LDS.  Contains a workgroup barrier: every thread of the workgroup must call it.
 __device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, const float* w, float4* xs_w, float* red, float eps, int K, int lane, int wave) {
-	n.w		= w;
-	n.xs_w	= xs_w;
-	n.scale = rms_scale_workgroup(rms_run_sumsq(x, K / GROUP_K, wave, lane), red, wave, lane, K, eps);
+	n.w		  = w;
+	n.xs_w	  = xs_w;
+	n.publish = nullptr;
+	n.epoch	  = 0;
+	n.scale	  = rms_scale_workgroup(rms_run_sumsq(x, K / GROUP_K, wave, lane), red, wave, lane, K, eps);
 }
 
 //
@@ -75,6 +85,8 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	int lane, int row, int N, bool dump_this_strip, unsigned epoch, gemv_norm* norm, int rowpart = 0, int spin_limit = PUBLISHED_SPIN_LIMIT) {
 	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
+	constexpr bool XPUB = XMODE == X_PUBLISHED || XMODE == X_PUBLISHED_EARLY; // the slice is read as tagged words
+	constexpr bool EARLY = XMODE == X_PUBLISHED_EARLY; // ... with a first look before the weight loads go out
 	static_assert(RS == 1 || RS == 2 || RS == 4, "a strip splits into 1, 2 or 4 row parts");
 	static_assert(RS == 1 || DUMP == DUMP_NONE, "the inspection variants run on whole strips");
 	constexpr int PART_ROWS = STRIP_ROWS / RS; // rows this workgroup owns
@@ -117,6 +129,21 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 		}
 	}
 
+	// device-scope loads: the producers ran on other XCDs, whose L2 this one does not snoop
+	constexpr int PW_LOADS = XPUB ? (TILES * GROUP_BLOCKS * PUBLISHED_WORDS + 63) / 64 : 1;
+	const uint64_t* pw	   = XPUB ? static_cast<const uint64_t*>(xin) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * PUBLISHED_WORDS) : nullptr;
+	const int n_words	   = cnt * GROUP_BLOCKS * PUBLISHED_WORDS;
+	uint64_t pv[PW_LOADS];
+	if constexpr (EARLY) {
+		// a first look ahead of the weight loads: a workgroup that starts after the publishers are through finds every word
+		// there and has its slice staged while its weights are still arriving
+#pragma unroll
+		for (int i = 0; i < PW_LOADS; ++i) {
+			const int v = lane + 64 * i;
+			pv[i]		= v < n_words ? __hip_atomic_load(pw + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : (static_cast<uint64_t>(epoch) << 32);
+		}
+	}
+
 	// ---- 2. every weight byte of the chunk, in flight at once ----
 	v4i q[TILES][W_LOADS];
 	v2u dd[TILES];
@@ -139,20 +166,19 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 
 	// ---- 2b. the slice comes from this launch's own producers: read it until every word is this launch's ----
 	bool timed_out = false;
-	if constexpr (XMODE == X_PUBLISHED) {
-		// device-scope loads: the producers ran on other XCDs, whose L2 this one does not snoop
-		const uint64_t* pw	   = static_cast<const uint64_t*>(xin) + static_cast<int64_t>(gc) * (GROUP_BLOCKS * PUBLISHED_WORDS);
-		constexpr int PW_LOADS = (TILES * GROUP_BLOCKS * PUBLISHED_WORDS + 63) / 64;
-		const int n_words	   = cnt * GROUP_BLOCKS * PUBLISHED_WORDS;
-		uint64_t pv[PW_LOADS];
-		int spins = 0;
+	if constexpr (XPUB) {
+		int spins	= 0;
+		bool looked = EARLY; // the first set of words is already on its way
 		for (;;) {
-			bool fresh = true;
+			if (!looked) {
 #pragma unroll
-			for (int i = 0; i < PW_LOADS; ++i) {
-				const int v = lane + 64 * i;
-				pv[i]		= v < n_words ? __hip_atomic_load(pw + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : (static_cast<uint64_t>(epoch) << 32);
+				for (int i = 0; i < PW_LOADS; ++i) {
+					const int v = lane + 64 * i;
+					pv[i]		= v < n_words ? __hip_atomic_load(pw + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : (static_cast<uint64_t>(epoch) << 32);
+				}
 			}
+			looked	   = false;
+			bool fresh = true;
 #pragma unroll
 			for (int i = 0; i < PW_LOADS; ++i) {
 				fresh = fresh && static_cast<unsigned>(pv[i] >> 32) == epoch;
@@ -237,6 +263,24 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	}
 	__builtin_amdgcn_wave_barrier(); // wave-local hand-off: the same wave wrote and reads; the LDS counter wait orders it
 
+	if constexpr (XF32 && NORM) {
+		if (norm->publish) {
+			// the slice as staged, for the workgroups that do not work it out themselves: self-tagged 64-bit words, device-scope
+			// stores, nothing waited for (a reader takes a word only with this launch's epoch in it)
+			uint64_t* out			= norm->publish + static_cast<int64_t>(gc) * (GROUP_BLOCKS * PUBLISHED_WORDS);
+			constexpr int OUT_WORDS = cnt * GROUP_BLOCKS * PUBLISHED_WORDS;
+#pragma unroll
+			for (int i = 0; i < (OUT_WORDS + 63) / 64; ++i) {
+				const int v = lane + 64 * i;
+				if (v < OUT_WORDS) {
+					const int blk		   = v / PUBLISHED_WORDS, j = v - blk * PUBLISHED_WORDS;
+					const uint32_t payload = j < 8 ? *reinterpret_cast<const uint32_t*>(xs_q + blk * QK + 4 * j) : __float_as_uint(xs_d[blk]);
+					__hip_atomic_store(out + v, (static_cast<uint64_t>(norm->epoch) << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				}
+			}
+		}
+	}
+
 	if constexpr (DUMP == DUMP_X) {
 		// parity hook: what was staged, written back as packed blocks (the first strip of the launch covers all of K)
 		if (dump_this_strip) {
@@ -288,7 +332,7 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 			}
 		}
 	}
-	if constexpr (XMODE == X_PUBLISHED) {
+	if constexpr (XPUB) {
 		if (timed_out) {
 			acc = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output as well
 		}
@@ -367,11 +411,20 @@ __device__ __forceinline__ void split_k_finish(uint64_t* __restrict__ tagged, un
 constexpr int GEMV_MAX_SPLIT_UNITS	= 8192; // strips * splits when splits > 1
 constexpr int GEMV_MAX_SPLIT_STRIPS = 512;
 constexpr int FFN_MAX_HIDDEN		= 65536; // rows of the gate / up projections in a fused FFN launch
+constexpr int GEMV_SHARED_X_MAX_K	= 65536; // longest input row that a launch with a norm shares between its workgroups (longer: each works it out)
+// Sharing makes every other workgroup wait for the first strip's: a chain of row read, norm, quantize, publish and read-back
+// of ~3 us that the first round of workgroups sits out.  It pays once a launch runs several rounds, each of which would
+// otherwise spend its first 1.5 us on the norm instead of on its loads: measured, lm_head [128256 x 4096] 88.6 -> 84.9 us,
+// gate+up [2 x 28672 x 8192] 84.1 -> 81.0 us, the one-launch FFN at those shapes 155 -> 133 us; but q+k+v [6144 x 4096]
+// 8.0 -> 9.6 us and nothing gained on gate+up [2 x 14336 x 4096] or its FFN (34.2 -> 34.0 us).
+constexpr int GEMV_SHARED_X_MIN_WORKGROUPS = 1024; // mat-vec launches
+constexpr int FFN_SHARED_X_MIN_PRODUCERS   = 768; // producer workgroups of a one-launch FFN
 struct gemv_scratch {
 	uint64_t* tagged   = nullptr; // [GEMV_MAX_SPLIT_UNITS][32] {epoch, partial sum}
 	float* gate_up	   = nullptr; // [2][FFN_MAX_HIDDEN]: the gate and up outputs (kept for inspection only)
 	uint64_t* act_words = nullptr; // [FFN_MAX_HIDDEN / 32][PUBLISHED_WORDS] {epoch, payload}: the quantized activation of the down projection
 	uint8_t* act_blocks = nullptr; // [FFN_MAX_HIDDEN / 32] packed 34-byte blocks: the activation of the three-launch form used under graph capture
+	uint64_t* x_words	= nullptr; // [GEMV_SHARED_X_MAX_K / 32][PUBLISHED_WORDS] {epoch, payload}: a launch's normalised, quantized input row, from its first strip's workgroups to the rest
 	unsigned epoch	   = 0; // with next_epoch = true: a value no earlier launch on this device has used
 	unsigned* error_word = nullptr; // 4 bytes of pinned host memory the device can write: non-zero once a kernel has given up a bounded wait
 	int spin_limit	   = PUBLISHED_SPIN_LIMIT; // polls before a consumer of published blocks gives up (lowered only by tests)

@@ -71,6 +71,44 @@ def test_norm_inside_the_one_launch_ffn(q8, oracle):
     assert rel_l2(to_host(y), oracle.gemv(wd, aq, n_out, n_ff)) <= 2e-6
 
 
+@pytest.mark.parametrize("ns,k", [([128256], 4096), ([8192], 28672), ([28672, 28672], 8192), ([32768, 1000, 33], 512)])
+def test_norm_row_shared_between_the_workgroups_of_a_large_launch(q8, oracle, ns, k):
+    # From 1024 workgroups on, only the first strip's workgroups (one per K split) normalise and quantize the row; they publish
+    # it and the rest read it.  The result must be the two-step form's (same quantized row, same mat-vec: bit for bit), on an
+    # unsplit launch, a K-split one, two and three matrices in one launch with ragged tails, and launch after launch with a new row.
+    wts = [q8.tile(q8.fill_weight_blocks(40 + i, n, k), n, k) for i, n in enumerate(ns)]
+    for rep in range(3):
+        x, w = row_inputs(50 + rep + k, 1, k, scale=1.0 + rep)
+        ys = q8.gemv_f32(wts if len(ns) > 1 else wts[0], to_dev(x[0]), ns if len(ns) > 1 else ns[0], k, norm_weight=to_dev(w), eps=EPS)
+        ys = ys if len(ns) > 1 else [ys]
+        xq = q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS)
+        assert np.array_equal(to_host(xq).reshape(-1), oracle.rms_norm_quantize_rows(x, w, EPS)[0].reshape(-1))
+        for i, n in enumerate(ns):
+            alone = to_host(q8.gemv(wts[i], xq.reshape(-1), n, k, True))
+            if len(ns) == 1:
+                assert np.array_equal(to_host(ys[i]), alone), (rep, i)  # one matrix: the stand-alone launch cuts K the same way
+            else:
+                assert rel_l2(to_host(ys[i]), alone) < 2e-6, (rep, i)  # a matrix launched alone may be cut differently: last bits
+
+
+def test_norm_row_shared_inside_the_one_launch_ffn(q8, oracle):
+    # 896 producer workgroups: the first publishes the normalised, quantized row, the others read it
+    n_ff, k, n_out = 28672, 1024, 256
+    wg_t, wu_t = (q8.tile(q8.fill_weight_blocks(60 + i, n_ff, k), n_ff, k) for i in range(2))
+    wd_t = q8.tile(q8.fill_weight_blocks(62, n_out, n_ff), n_out, n_ff)
+    for rep in range(3):
+        x, w = row_inputs(70 + rep, 1, k, scale=0.5 + rep)
+        y = q8.ffn(wg_t, wu_t, wd_t, to_dev(x[0]), n_ff, k, n_out, norm_weight=to_dev(w), eps=EPS)
+        g, u = q8.debug_ffn_gate_up(n_ff)
+        xq = q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS)
+        # gate and up are mat-vecs of the same quantized row: the stand-alone kernel cuts K differently, so last bits may differ
+        assert rel_l2(to_host(g), to_host(q8.gemv(wg_t, xq.reshape(-1), n_ff, k, True))) < 2e-6
+        assert rel_l2(to_host(u), to_host(q8.gemv(wu_t, xq.reshape(-1), n_ff, k, True))) < 2e-6
+        aq = oracle.silu_mul_quantize_rows(to_host(g), to_host(u))[0]
+        rows = 64
+        assert rel_l2(to_host(y)[:rows], oracle.gemv(oracle.fill_weights(62, rows, n_ff), aq, rows, n_ff)) <= REL_L2_TOL
+
+
 def test_rms_norm_errors(q8):
     import torch
 
