@@ -48,10 +48,14 @@ struct ffn_args {
 	uint64_t* x_words; // scratch (NORM): the normalised, quantized input row, published by the first producer workgroup for the others; null: each works it out
 };
 
-template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
+// PAIR: every producer wave takes a K range of BOTH matrices (the strip's rows of gate and of up against one staged slice of
+// the input row), sixteen ranges per workgroup, instead of eight waves per matrix each staging the same eight slices: the row
+// (and the norm weights) are fetched and quantized once per workgroup instead of twice.  For K up to 2 groups per wave.
+template<int TILES, bool LOOP, bool NORM, bool PAIR = false> __global__ __launch_bounds__(GEMV_WAVES * 64) void ffn_decode_kernel(ffn_args a) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][TILES * GROUP_K];
 	__shared__ float xs_d[GEMV_WAVES][TILES * GROUP_BLOCKS];
 	__shared__ float red[GEMV_WAVES][64];
+	__shared__ float red_up[PAIR ? GEMV_WAVES : 1][64];
 
 	const int tid  = threadIdx.x;
 	const int lane = tid & 63;
@@ -63,16 +67,21 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 		__shared__ __align__(16) float act_f[STRIP_ROWS];
 		__shared__ float norm_red[16];
 		__shared__ float4 xs_w[NORM ? GEMV_WAVES : 1][NORM ? TILES * 32 : 1];
-		const int matrix	   = wave >> 3;
-		const int slot		   = wave & 7;
+		const int matrix	   = PAIR ? 0 : wave >> 3;
+		const int slot		   = PAIR ? wave : wave & 7;
 		const int strip		   = wg;
 		const int g0		   = slot * a.p_per_slot + min(slot, a.p_rem);
 		const int g1		   = g0 + a.p_per_slot + (slot < a.p_rem ? 1 : 0);
 		const uint8_t* w_strip = (matrix ? a.w_up : a.w_gate) + macro_offset(strip, 0, a.groups_p);
+		const uint8_t* w_other = PAIR ? a.w_up + macro_offset(strip, 0, a.groups_p) : nullptr;
 		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
 		float acc			   = 0.0f;
+		[[maybe_unused]] float acc_up = 0.0f;
 		auto walk = [&]<int XMODE, bool WITH_NORM>(const void* x_from, void* dump_to, gemv_norm* norm) {
-			if constexpr (!LOOP) {
+			if constexpr (PAIR) {
+				return gemv_chunk<2, XMODE, DUMP_NONE, WITH_NORM, 1, 2>(w_strip, x_from, dump_to, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, a.epoch, norm, 0, a.spin_limit,
+					w_other, &acc_up);
+			} else if constexpr (!LOOP) {
 				return gemv_chunk<TILES, XMODE, DUMP_NONE, WITH_NORM>(w_strip, x_from, dump_to, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, a.epoch, norm, 0, a.spin_limit);
 			} else {
 				float sum = 0.0f;
@@ -96,6 +105,8 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 			} else {
 				acc = walk.template operator()<X_PUBLISHED_EARLY, false>(a.x_words, a.error_word, nullptr);
 			}
+		} else if constexpr (PAIR) {
+			acc = walk.template operator()<X_F32, false>(a.x, nullptr, nullptr);
 		} else if constexpr (!LOOP) {
 			acc = gemv_chunk<TILES, X_F32, DUMP_NONE, false>(w_strip, a.x, nullptr, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_p, lane, row_l, a.n_ff, false, 0, nullptr);
 		} else {
@@ -104,15 +115,26 @@ template<int TILES, bool LOOP, bool NORM> __global__ __launch_bounds__(GEMV_WAVE
 				__builtin_amdgcn_wave_barrier();
 			}
 		}
+		if constexpr (PAIR) {
+			red_up[wave][lane] = acc_up;
+		}
 		red[wave][lane] = acc;
 		__syncthreads();
 		if (wave == 0) {
 			if (lane < STRIP_ROWS) {
 				float g = 0.0f, u = 0.0f;
+				if constexpr (PAIR) {
 #pragma unroll
-				for (int w = 0; w < GEMV_WAVES / 2; ++w) {
-					g += red[w][lane] + red[w][32 + lane];
-					u += red[GEMV_WAVES / 2 + w][lane] + red[GEMV_WAVES / 2 + w][32 + lane];
+					for (int w = 0; w < GEMV_WAVES; ++w) {
+						g += red[w][lane] + red[w][32 + lane];
+						u += red_up[w][lane] + red_up[w][32 + lane];
+					}
+				} else {
+#pragma unroll
+					for (int w = 0; w < GEMV_WAVES / 2; ++w) {
+						g += red[w][lane] + red[w][32 + lane];
+						u += red[GEMV_WAVES / 2 + w][lane] + red[GEMV_WAVES / 2 + w][32 + lane];
+					}
 				}
 				act_f[lane]									 = silu_mul(g, u);
 				a.gate_up[strip * STRIP_ROWS + lane]				 = g; // inspection copies, not read by this launch
@@ -184,11 +206,11 @@ __global__ void ffn_empty_kernel(float* __restrict__ y, const float* __restrict_
 	}
 }
 
-template<int TILES, bool LOOP> static hipError_t launch_ffn_t(const ffn_args& a, unsigned grid, hipStream_t s) {
+template<int TILES, bool LOOP, bool PAIR = false> static hipError_t launch_ffn_t(const ffn_args& a, unsigned grid, hipStream_t s) {
 	if (a.norm_w) {
-		return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP, true>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
+		return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP, true, PAIR>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
 	}
-	return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP, false>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
+	return launch_kernel(KIND_GEMV, ffn_decode_kernel<TILES, LOOP, false, PAIR>, dim3(grid), dim3(GEMV_WAVES * 64), 0, s, a);
 }
 
 // n_ff % 128 == 0, K % 128 == 0, n_ff <= FFN_MAX_HIDDEN (checked by the caller).
@@ -256,17 +278,28 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	a.groups_c	 = groups_c;
 	a.producers	 = static_cast<int>(n_ff / STRIP_ROWS);
 	a.x_words	 = norm_w && a.producers >= FFN_SHARED_X_MIN_PRODUCERS && K <= GEMV_SHARED_X_MAX_K ? sc.x_words : nullptr;
-	a.p_per_slot = a.groups_p / (GEMV_WAVES / 2);
-	a.p_rem		 = a.groups_p % (GEMV_WAVES / 2);
+	// up to two groups per wave when the row is cut sixteen ways: every producer wave takes both matrices (PAIR)
+	// ... where the eight-and-eight form would need the four-group kernel anyway (the two-group kernel fits two workgroups per
+	// CU and is left alone), and not with the chunked walk
+	const int tiles_8_8 = (a.groups_p + GEMV_WAVES / 2 - 1) / (GEMV_WAVES / 2);
+	// Measured at the LLaMA-3-8B shapes: with the norm in front 34.2 -> 33.1 us (the row AND the norm weights once instead of twice
+	// per workgroup), without it 31.2 -> 31.3 us (the row alone stays in the CU's L1 between the two halves): used with a norm only.
+	const bool pair		= norm_w && (a.groups_p + GEMV_WAVES - 1) / GEMV_WAVES <= 2 && tiles_for(splits) <= 4 && (tiles_8_8 > 2 || tiles_for(splits) > 2);
+	const int p_slots  = pair ? GEMV_WAVES : GEMV_WAVES / 2;
+	a.p_per_slot	   = a.groups_p / p_slots;
+	a.p_rem			   = a.groups_p % p_slots;
 	int shift	 = 0;
 	while ((1 << shift) < splits) {
 		++shift;
 	}
 	a.split_shift		= shift;
-	const int tiles_p	= (a.groups_p + GEMV_WAVES / 2 - 1) / (GEMV_WAVES / 2);
+	const int tiles_p	= pair ? 2 : (a.groups_p + GEMV_WAVES / 2 - 1) / (GEMV_WAVES / 2); // LDS slice per wave, in groups
 	const int tiles_c	= tiles_for(splits);
 	const int tiles		= tiles_p > tiles_c ? tiles_p : tiles_c;
 	const unsigned grid = static_cast<unsigned>(a.producers + strips_c * splits);
+	if (pair) {
+		return launch_ffn_t<4, false, true>(a, grid, s);
+	}
 	if (tiles > 4) {
 		return launch_ffn_t<4, true>(a, grid, s);
 	}

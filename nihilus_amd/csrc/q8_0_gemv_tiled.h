@@ -80,9 +80,14 @@ __device__ __forceinline__ void gemv_norm_begin(gemv_norm& n, const float* x, co
 // blocks instead of one (a group takes 4 / RS loads per lane) and the lane's block and half follow from its number.
 // A matrix with fewer strips than the chip has CUs spreads over RS times as many of them this way, with nothing to
 // hand over between workgroups.
-template<int TILES, int XMODE, int DUMP, bool NORM, int CNT, int RS = 1>
+// MATS == 2: two weight strips (w_strip, w_strip2: the same rows of two matrices that share the activation, gate and up)
+// against ONE staged slice: the slice is fetched, quantized and read back from LDS once for both; the second matrix's
+// sum comes back through acc2.
+template<int TILES, int XMODE, int DUMP, bool NORM, int CNT, int RS = 1, int MATS = 1>
 __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int groups,
-	int lane, int row, int N, bool dump_this_strip, unsigned epoch, gemv_norm* norm, int rowpart = 0, int spin_limit = PUBLISHED_SPIN_LIMIT) {
+	int lane, int row, int N, bool dump_this_strip, unsigned epoch, gemv_norm* norm, int rowpart = 0, int spin_limit = PUBLISHED_SPIN_LIMIT, const uint8_t* __restrict__ w_strip2 = nullptr,
+	float* acc2 = nullptr) {
+	static_assert(MATS == 1 || (MATS == 2 && RS == 1 && DUMP == DUMP_NONE), "two matrices: whole strips, production form");
 	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
 	constexpr bool XPUB = XMODE == X_PUBLISHED || XMODE == X_PUBLISHED_EARLY; // the slice is read as tagged words
@@ -160,6 +165,22 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 					q[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * (RS * TILE_BYTES) + lane_off));
 				}
 				dd[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
+			}
+		}
+	}
+	v4i q2[MATS == 2 ? TILES : 1][W_LOADS];
+	v2u dd2[MATS == 2 ? TILES : 1];
+	if constexpr (MATS == 2) {
+		const uint8_t* macro0 = w_strip2 + static_cast<int64_t>(gc) * MACRO_BYTES;
+#pragma unroll
+		for (int t = 0; t < TILES; ++t) {
+			if (t < cnt) {
+				const uint8_t* macro = macro0 + t * MACRO_BYTES;
+#pragma unroll
+				for (int j = 0; j < W_LOADS; ++j) {
+					q2[t][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(macro + j * TILE_BYTES + 16 * lane));
+				}
+				dd2[t] = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(macro + MACRO_D_OFFSET + 8 * r));
 			}
 		}
 	}
@@ -298,6 +319,7 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 
 	// ---- 4. dot products as the tiles land ----
 	float acc = 0.0f;
+	[[maybe_unused]] float second = 0.0f;
 #pragma unroll
 	for (int t = 0; t < TILES; ++t) {
 		if (t < cnt) {
@@ -317,6 +339,11 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 					} else {
 						acc = fmaf(static_cast<float>(s), dw[j] * xs_d[jj], acc);
 					}
+					if constexpr (MATS == 2) {
+						const uint32_t dp2 = (j & 2) ? dd2[t].y : dd2[t].x;
+						const float dw2	   = half_bits_to_float(static_cast<uint16_t>((j & 1) ? (dp2 >> 16) : (dp2 & 0xFFFFu)));
+						second			   = fmaf(static_cast<float>(dot16(q2[t][j], xv)), dw2 * xs_d[jj], second);
+					}
 				}
 			} else {
 #pragma unroll
@@ -334,19 +361,25 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	}
 	if constexpr (XPUB) {
 		if (timed_out) {
-			acc = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output as well
+			acc	   = __uint_as_float(0x7FC00000u); // a producer never published: make the failure visible in the output as well
+			second = acc;
 		}
+	}
+	if constexpr (MATS == 2) {
+		*acc2 = second;
 	}
 	return acc;
 }
 
-template<int TILES, int XMODE, int DUMP, bool NORM = false, int RS = 1>
+template<int TILES, int XMODE, int DUMP, bool NORM = false, int RS = 1, int MATS = 1>
 __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip, const void* __restrict__ xin, void* __restrict__ dump, uint8_t* xs_q, float* xs_d, int gc, int cnt,
-	int groups, int lane, int row, int N, bool dump_this_strip, unsigned epoch = 0, gemv_norm* norm = nullptr, int rowpart = 0, int spin_limit = PUBLISHED_SPIN_LIMIT) {
+	int groups, int lane, int row, int N, bool dump_this_strip, unsigned epoch = 0, gemv_norm* norm = nullptr, int rowpart = 0, int spin_limit = PUBLISHED_SPIN_LIMIT,
+	const uint8_t* __restrict__ w_strip2 = nullptr, float* acc2 = nullptr) {
 #define NH_CHUNK_CASE(C)                                                                                                                                              \
 	case C:                                                                                                                                                           \
 		if constexpr (C <= TILES) {                                                                                                                                   \
-			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0), RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart, spin_limit); \
+			return gemv_chunk_n<TILES, XMODE, DUMP, NORM, (C <= TILES ? C : 0), RS, MATS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart,   \
+				spin_limit, w_strip2, acc2);                                                                                                                          \
 		}                                                                                                                                                             \
 		break;
 	switch (cnt) { // wave-uniform
@@ -358,7 +391,8 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 			break;
 	}
 #undef NH_CHUNK_CASE
-	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0, RS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart, spin_limit); // an idle wave (still takes part in barriers)
+	// an idle wave (still takes part in barriers)
+	return gemv_chunk_n<TILES, XMODE, DUMP, NORM, 0, RS, MATS>(w_strip, xin, dump, xs_q, xs_d, gc, groups, lane, row, N, dump_this_strip, epoch, norm, rowpart, spin_limit, w_strip2, acc2);
 }
 
 // K split over several workgroups: each publishes the 32 partial sums of its share, tagged with the launch's epoch
