@@ -109,6 +109,29 @@ def test_norm_row_shared_inside_the_one_launch_ffn(q8, oracle):
         assert rel_l2(to_host(y)[:rows], oracle.gemv(oracle.fill_weights(62, rows, n_ff), aq, rows, n_ff)) <= REL_L2_TOL
 
 
+@pytest.mark.parametrize("n_ff,k,n_out", [(4096, 3072, 256), (2048, 2560, 512), (14336, 4096, 4096)])
+def test_norm_ffn_with_producer_waves_on_both_matrices(q8, oracle, n_ff, k, n_out):
+    # K of 17..32 groups with a norm: the producer workgroup cuts the row sixteen ways and every wave takes its range of gate AND
+    # up against one staged slice (ranges of one and two groups mixed when K / 128 is not a multiple of 16)
+    wg_t, wu_t = (q8.tile(q8.fill_weight_blocks(80 + i, n_ff, k), n_ff, k) for i in range(2))
+    wd_t = q8.tile(q8.fill_weight_blocks(82, n_out, n_ff), n_out, n_ff)
+    x, w = row_inputs(n_ff + k, 1, k, scale=0.7)
+    res = np.random.default_rng(1).standard_normal(n_out).astype(np.float32)
+    y = q8.ffn(wg_t, wu_t, wd_t, to_dev(x[0]), n_ff, k, n_out, residual=to_dev(res), norm_weight=to_dev(w), eps=EPS)
+    g, u = q8.debug_ffn_gate_up(n_ff)
+    xq = oracle.rms_norm_quantize_rows(x, w, EPS)[0]
+    rows = min(n_ff, 256)
+    assert rel_l2(to_host(g)[:rows], oracle.gemv(oracle.fill_weights(80, rows, k), xq, rows, k)) <= REL_L2_TOL
+    assert rel_l2(to_host(u)[:rows], oracle.gemv(oracle.fill_weights(81, rows, k), xq, rows, k)) <= REL_L2_TOL
+    xq_d = q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS)
+    assert rel_l2(to_host(g), to_host(q8.gemv(wg_t, xq_d.reshape(-1), n_ff, k, True))) < 2e-6  # every row, against the stand-alone mat-vec
+    assert rel_l2(to_host(u), to_host(q8.gemv(wu_t, xq_d.reshape(-1), n_ff, k, True))) < 2e-6
+    aq = oracle.silu_mul_quantize_rows(to_host(g), to_host(u))[0]
+    rows_out = min(n_out, 64)
+    assert rel_l2(to_host(y)[:rows_out], oracle.gemv(oracle.fill_weights(82, rows_out, n_ff), aq, rows_out, n_ff) + res[:rows_out]) <= REL_L2_TOL
+    assert np.array_equal(to_host(q8.ffn(wg_t, wu_t, wd_t, to_dev(x[0]), n_ff, k, n_out, residual=to_dev(res), norm_weight=to_dev(w), eps=EPS)), to_host(y))  # bit-stable
+
+
 def test_rms_norm_errors(q8):
     import torch
 
