@@ -200,7 +200,10 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	int groups) {
 	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
 	constexpr int STAGE_BYTES = DATA_BYTES + 16;
-	__shared__ __align__(16) uint8_t lds_all[KS][2 * STAGE_BYTES + 256]; // + 256: where waves that copy no scale table put theirs
+	constexpr int SET_BYTES	   = 2 * STAGE_BYTES + 256; // + 256: where waves that copy no scale table put theirs
+	constexpr int PARK_BYTES   = KS > 1 ? KS * 4 * (KS - 1) * (16 * TM / KS) * 64 * 4 : 0; // the final sum over the K sets, below
+	constexpr int LDS_BYTES	   = KS * SET_BYTES > PARK_BYTES ? KS * SET_BYTES : PARK_BYTES;
+	__shared__ __align__(16) uint8_t lds_raw[LDS_BYTES];
 	typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 	typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -209,7 +212,7 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wave	   = wave_all & 3; // which of the workgroup's four weight strips
 	const int kr	   = wave_all >> 2; // which K range
-	uint8_t* lds	   = lds_all[kr];
+	uint8_t* lds	   = lds_raw + kr * SET_BYTES;
 	const int g_len	   = groups / KS; // the host launches KS > 1 only when it divides
 	const int g_base   = kr * g_len;
 	const int half	   = lane >> 5;
@@ -279,6 +282,23 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		}
 		r.d = load_sv<v2u, STREAM>(scalar_base(W, at + MACRO_D_OFFSET), l8);
 	};
+	// load number p of a group's set (PIECES of them: TM activation tiles, their scale dword, four weight tiles, their scales);
+	// the same loads as fetch_a and fetch_w, which the prologue issues in one go
+	constexpr int PIECES = TM + 2 + GROUP_BLOCKS;
+	auto fetch_piece = [&](int p, int g, a_regs& ra, w_regs& rw) {
+		uint32_t l16 = lane16;
+		asm volatile("" : "+v"(l16));
+		if (p < TM) {
+			ra.q[p] = load_sv<v4i, false>(scalar_base(A, a_off[p] + static_cast<int64_t>(g) * MACRO_BYTES), l16);
+		} else if (p == TM) {
+			ra.d = load_sv<uint32_t, false>(scalar_base(A, sc_off + static_cast<int64_t>(g) * MACRO_BYTES), l16 >> 2);
+		} else if (p < TM + 1 + GROUP_BLOCKS) {
+			const int k = p - TM - 1;
+			rw.q[k] = load_sv<v4i, STREAM>(scalar_base(W, w_off + static_cast<int64_t>(g) * MACRO_BYTES + k * TILE_BYTES), l16);
+		} else {
+			rw.d = load_sv<v2u, STREAM>(scalar_base(W, w_off + static_cast<int64_t>(g) * MACRO_BYTES + MACRO_D_OFFSET), (l16 & 0x1F0u) >> 1);
+		}
+	};
 	v16f acc[TM];
 #pragma unroll
 	for (int i = 0; i < TM; ++i) {
@@ -293,15 +313,16 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	fetch_w(0, wa);
 	stash_a(0, pre);
 	__syncthreads();
-	// One trip = one 128-quant group.  Requested at its start: the next group's activation tiles, then its weight tiles -- in
+	// One trip = one 128-quant group.  Requested during it: the next group's activation tiles, then its weight tiles -- in
 	// that order, because loads return in issue order: the (cached) activations are needed at the trip's end, for the barrier,
-	// and must not queue behind weights that have until the next trip to arrive.  Past the end the last group is requested
-	// again (a cache hit that nobody uses): every trip issues the same loads, so every wait the compiler places is a count
-	// (a load under a condition makes it wait for everything outstanding instead).
+	// and must not queue behind weights that have until the next trip to arrive.  The requests are spread over the trip's
+	// units, one or two behind each unit's LDS read: issued together at the trip's start, the sixteen waves of a CU that
+	// leave the barrier at the same moment queue at the memory pipeline (0.4 to 2 k cycles per wave and trip before its first
+	// MFMA).  Past the end the last group is requested again (a cache hit that nobody uses): every trip issues the same
+	// loads, so every wait the compiler places is a count (a load under a condition makes it wait for everything
+	// outstanding instead).
 	auto trip = [&](int g, w_regs& cur, w_regs& nxt) {
-		fetch_a(min(g + 1, last), pre);
-		fetch_w(min(g + 1, last), nxt);
-		__builtin_amdgcn_sched_barrier(0);
+		const int gn = min(g + 1, last);
 		if (half) {
 			cur.d = v2u{ 0u, 0u };
 		}
@@ -323,6 +344,11 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 			uint32_t s_nxt	= s_cur;
 			if (u + 1 < UNITS) {
 				read_a(u + 1, a_nxt, s_nxt);
+			}
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for (int pc = u * PIECES / UNITS; pc < (u + 1) * PIECES / UNITS; ++pc) {
+				fetch_piece(pc, gn, pre, nxt);
 			}
 			__builtin_amdgcn_sched_barrier(0);
 			const uint32_t wd = (t < 2) ? cur.d.x : cur.d.y;
@@ -362,38 +388,55 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		}
 	}
 	if constexpr (KS > 1 && !DUMP) {
-		// sets 1 .. KS-1 park their tiles one after the other in the same LDS buffer, set 0 adds them (set order, fixed)
-		static_assert(sizeof(lds_all) >= 4 * TM * 16 * 64 * sizeof(float), "the stages double as the reduction buffer");
+		// The K sets' tiles are summed by all of them at once: set q keeps PER = 16 / KS of a lane's 16 values per strip (with
+		// four sets: rows 8q .. 8q+7 of every 32-row strip), parks the other sets' shares in LDS, and after one barrier adds what
+		// the others parked for it, in set order (s0 + s1 + s2 + s3 whatever q is, so the result does not depend on who adds),
+		// and stores its own rows.  One set adding the others' whole tiles in turn took 12 % of the launch at M=512, N=K=4096.
+		constexpr int PER = 16 / KS;
 		__syncthreads(); // every set is through with its stages
-		float* slot = reinterpret_cast<float*>(&lds_all[0][0]) + wave * (TM * 16 * 64);
+		float* park = reinterpret_cast<float*>(lds_raw);
+		auto slot	= [&](int q, int src) { // where set src parks its share of part q (src != q), this wave's strip
+			return park + ((((q * 4 + wave) * (KS - 1)) + (src < q ? src : src - 1)) * (PER * TM)) * 64 + lane;
+		};
 #pragma unroll
-		for (int k = 1; k < KS; ++k) {
-			if (kr == k) {
-#pragma unroll
-				for (int i = 0; i < TM; ++i) {
-#pragma unroll
-					for (int e = 0; e < 16; ++e) {
-						slot[(i * 16 + e) * 64 + lane] = acc[i][e];
-					}
-				}
-			}
-			__syncthreads();
-			if (kr == 0) {
+		for (int q = 0; q < KS; ++q) {
+			if (q != kr) {
+				float* dst = slot(q, kr);
 #pragma unroll
 				for (int i = 0; i < TM; ++i) {
 #pragma unroll
-					for (int e = 0; e < 16; ++e) {
-						acc[i][e] += slot[(i * 16 + e) * 64 + lane];
+					for (int e = 0; e < PER; ++e) {
+						dst[(i * PER + e) * 64] = acc[i][q * PER + e];
 					}
 				}
 			}
-			if (k + 1 < KS) {
-				__syncthreads();
+		}
+		__syncthreads();
+		const int n = ns * 32 + (lane & 31);
+#pragma unroll
+		for (int q = 0; q < KS; ++q) {
+			if (q == kr) {
+#pragma unroll
+				for (int i = 0; i < TM; ++i) {
+#pragma unroll
+					for (int e = 0; e < PER; ++e) {
+						float v = 0.0f;
+#pragma unroll
+						for (int src = 0; src < KS; ++src) {
+							const float part = src == q ? acc[i][q * PER + e] : slot(q, src)[(i * PER + e) * 64];
+							v				 = src == 0 ? part : v + part;
+						}
+						const int ee = q * PER + e;
+						const int m	 = (ms0 + i) * 32 + 8 * (ee >> 2) + 4 * half + (ee & 3);
+						if (m < M && n < N) {
+							const int64_t at = static_cast<int64_t>(m) * N + n;
+							C[at]			 = R ? v + R[at] : v; // R may be C: read before the write, by the same thread
+						}
+					}
+				}
 			}
 		}
-		if (kr > 0) {
-			return;
-		}
+		return;
 	}
 	if constexpr (!DUMP) {
 		const int n = ns * 32 + (lane & 31);
