@@ -306,6 +306,9 @@ constexpr int64_t GEMM_SKINNY_MAX_M = 64;
 // Make this device's K-split scratch buffers now (otherwise: on the first launch that needs one).
 hipError_t prepare_gemv_scratch();
 hipError_t prepare_gemm_scratch();
+constexpr int64_t GEMM_SPLIT_SCRATCH_FLOATS = 2048 * 2 * 16 * 64; // partial tiles of a K split over workgroups
+constexpr int GEMM_SPLIT_MAX_UNITS			  = 512; // arrival counters
+hipError_t acquire_gemm_split_scratch(float** partials, unsigned** counters, hipStream_t s);
 hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual = nullptr);
 
 } // namespace nh

@@ -23,6 +23,7 @@ constexpr int GEMM_TN	   = 2; // along N
 constexpr int GEMM_BM	   = GEMM_WAVES_M * GEMM_TM * 32; // 128
 constexpr int GEMM_BN	   = GEMM_WAVES_N * GEMM_TN * 32; // 128
 constexpr int GEMM_THREADS = GEMM_WAVES_M * GEMM_WAVES_N * 64;
+constexpr int GEMM_SPLIT_MIN_TRIPS = 2; // K goes over more workgroups only while each K set keeps this many 128-quant groups
 constexpr int GEMM_STREAM_TILE_MIN_COLUMN_BLOCKS = 192; // 128-row column blocks from which the tile kernel also takes the few-row (batched decode) shapes
 
 // 16 operand bytes for (row strip, block b): lane supplies row strip*32 + lane%32, half lane/32.
@@ -195,9 +196,10 @@ template<typename T, bool NT> __device__ __forceinline__ T load_sv(gptr_u8 p, ui
 	}
 }
 
-template<int TM, bool DUMP, int KS = 1, bool STREAM = false>
+template<int TM, bool DUMP, int KS = 1, bool STREAM = false, bool SPLIT = false>
 __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* C, const float* R, int32_t* __restrict__ sums, int M, int N,
-	int groups) {
+	int groups, float* __restrict__ partials = nullptr, unsigned* __restrict__ counters = nullptr) {
+	static_assert(!SPLIT || (KS > 1 && !DUMP), "K over several workgroups continues the K sets' sum");
 	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
 	constexpr int STAGE_BYTES = DATA_BYTES + 16;
 	constexpr int SET_BYTES	   = 2 * STAGE_BYTES + 256; // + 256: where waves that copy no scale table put theirs
@@ -213,8 +215,9 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	const int wave	   = wave_all & 3; // which of the workgroup's four weight strips
 	const int kr	   = wave_all >> 2; // which K range
 	uint8_t* lds	   = lds_raw + kr * SET_BYTES;
-	const int g_len	   = groups / KS; // the host launches KS > 1 only when it divides
-	const int g_base   = kr * g_len;
+	// the host launches KS > 1, and K over gridDim.z workgroups, only when they divide
+	const int g_len	   = SPLIT ? groups / (KS * static_cast<int>(gridDim.z)) : groups / KS;
+	const int g_base   = SPLIT ? (static_cast<int>(blockIdx.z) * KS + kr) * g_len : kr * g_len;
 	const int half	   = lane >> 5;
 	const int m_strips = (M + 31) / 32;
 	const int n_strips = (N + 31) / 32;
@@ -413,6 +416,7 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		}
 		__syncthreads();
 		const int n = ns * 32 + (lane & 31);
+		float mine[TM * PER]; // this wave's rows of the workgroup's tile (SPLIT: of its share of K)
 #pragma unroll
 		for (int q = 0; q < KS; ++q) {
 			if (q == kr) {
@@ -426,13 +430,64 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 							const float part = src == q ? acc[i][q * PER + e] : slot(q, src)[(i * PER + e) * 64];
 							v				 = src == 0 ? part : v + part;
 						}
-						const int ee = q * PER + e;
-						const int m	 = (ms0 + i) * 32 + 8 * (ee >> 2) + 4 * half + (ee & 3);
-						if (m < M && n < N) {
-							const int64_t at = static_cast<int64_t>(m) * N + n;
-							C[at]			 = R ? v + R[at] : v; // R may be C: read before the write, by the same thread
-						}
+						mine[i * PER + e] = v;
 					}
+				}
+			}
+		}
+		if constexpr (SPLIT) {
+			// K over gridDim.z workgroups: every one leaves its tile in the scratch (each wave its own rows, as it holds them),
+			// counts itself in, and the last to arrive adds the tiles in z order -- whoever that is -- and stores
+			__shared__ int last_flag;
+			const int kz_count = static_cast<int>(gridDim.z);
+			const int unit	   = static_cast<int>(blockIdx.y * gridDim.x + blockIdx.x);
+			constexpr int TILE_FLOATS = 4 * KS * TM * PER * 64; // = TM * 4096: a workgroup's tile
+			float* tile = partials + (static_cast<int64_t>(unit) * kz_count) * TILE_FLOATS + wave_all * (TM * PER * 64) + lane;
+			float* dst	= tile + static_cast<int64_t>(blockIdx.z) * TILE_FLOATS;
+#pragma unroll
+			for (int j = 0; j < TM * PER; ++j) {
+				__hip_atomic_store(&dst[j * 64], mine[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
+			wait_stores_acknowledged();
+			__syncthreads();
+			if (tid == 0) {
+				const unsigned prev = __hip_atomic_fetch_add(&counters[unit], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				const int last		= (prev == static_cast<unsigned>(kz_count - 1));
+				if (last) {
+					__hip_atomic_store(&counters[unit], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
+				}
+				last_flag = last;
+			}
+			__syncthreads();
+			if (!last_flag) {
+				return;
+			}
+#pragma unroll
+			for (int j = 0; j < TM * PER; ++j) {
+				mine[j] = 0.0f;
+			}
+			for (int z = 0; z < kz_count; ++z) {
+				float got[TM * PER];
+#pragma unroll
+				for (int j = 0; j < TM * PER; ++j) {
+					got[j] = __hip_atomic_load(&tile[static_cast<int64_t>(z) * TILE_FLOATS + j * 64], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				}
+#pragma unroll
+				for (int j = 0; j < TM * PER; ++j) {
+					mine[j] = z == 0 ? got[j] : mine[j] + got[j];
+				}
+			}
+		}
+#pragma unroll
+		for (int i = 0; i < TM; ++i) {
+#pragma unroll
+			for (int e = 0; e < PER; ++e) {
+				const int ee = kr * PER + e;
+				const int m	 = (ms0 + i) * 32 + 8 * (ee >> 2) + 4 * half + (ee & 3);
+				if (m < M && n < N) {
+					const int64_t at = static_cast<int64_t>(m) * N + n;
+					const float v	 = mine[i * PER + e];
+					C[at]			 = R ? v + R[at] : v; // R may be C: read before the write, by the same thread
 				}
 			}
 		}
@@ -459,7 +514,7 @@ template<int TM, bool STREAM> static hipError_t launch_gemm_tiled_t(const uint8_
 	const int m_strips = (m + 31) / 32, n_strips = (n + 31) / 32;
 	const dim3 grid(static_cast<unsigned>((n_strips + 3) / 4), static_cast<unsigned>((m_strips + TM - 1) / TM));
 	if (sums) {
-		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, R, sums, m, n, groups);
+		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, R, sums, m, n, groups, nullptr, nullptr);
 		return hipGetLastError();
 	}
 	// a grid that leaves SIMDs short of their four waves: K sets inside the workgroup (8 or 16 waves) make up for it
@@ -467,13 +522,32 @@ template<int TM, bool STREAM> static hipError_t launch_gemm_tiled_t(const uint8_
 	while (ks < 4 && static_cast<int64_t>(grid.x) * grid.y * 4 * ks * 2 <= 4096 && groups % (ks * 2) == 0 && groups / (ks * 2) >= 4) {
 		ks *= 2;
 	}
+	if constexpr (STREAM) {
+		// still short of one workgroup per CU: K over kz workgroups per tile as well, their tiles added through the scratch
+		const int64_t wgs = static_cast<int64_t>(grid.x) * grid.y;
+		int kz = 1;
+		while (ks == 4 && wgs * kz * 2 <= 256 && groups % (ks * kz * 2) == 0 && groups / (ks * kz * 2) >= GEMM_SPLIT_MIN_TRIPS && wgs * kz * 2 * TM * 4096 <= GEMM_SPLIT_SCRATCH_FLOATS &&
+			wgs <= GEMM_SPLIT_MAX_UNITS) {
+			kz *= 2;
+		}
+		if (kz > 1) {
+			float* partials	   = nullptr;
+			unsigned* counters = nullptr;
+			const hipError_t e = acquire_gemm_split_scratch(&partials, &counters, s);
+			if (e != hipSuccess) {
+				return e;
+			}
+			return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4, true, true>, dim3(grid.x, grid.y, static_cast<unsigned>(kz)), dim3(1024), 0, s, w, a, C, R, sums, m, n, groups, partials,
+				counters);
+		}
+	}
 	if (ks == 4) {
-		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4, STREAM>, grid, dim3(1024), 0, s, w, a, C, R, sums, m, n, groups);
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4, STREAM>, grid, dim3(1024), 0, s, w, a, C, R, sums, m, n, groups, static_cast<float*>(nullptr), static_cast<unsigned*>(nullptr));
 	}
 	if (ks == 2) {
-		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2, STREAM>, grid, dim3(512), 0, s, w, a, C, R, sums, m, n, groups);
+		return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 2, STREAM>, grid, dim3(512), 0, s, w, a, C, R, sums, m, n, groups, static_cast<float*>(nullptr), static_cast<unsigned*>(nullptr));
 	}
-	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 1, STREAM>, grid, dim3(256), 0, s, w, a, C, R, sums, m, n, groups);
+	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 1, STREAM>, grid, dim3(256), 0, s, w, a, C, R, sums, m, n, groups, static_cast<float*>(nullptr), static_cast<unsigned*>(nullptr));
 }
 
 // Two activation strips per wave whenever there are two: every weight tile fetched is used twice, which halves what a CU
@@ -522,6 +596,15 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 		// in is what bounds both kernels ([28672 x 8192] at M = 16 / 32 / 64: 50 / 55 / 75 us streaming, 44 / 44 / 69 us
 		// here; [128256 x 8192]: 193 / - / 298 against 182 / - / 221 us).  Below that the tile kernel's grid leaves CUs idle
 		// ([14336 x 4096] at M = 64: 30 us against 23 us) and the streaming kernel, which can split K over workgroups, stays.
+		// Between the two, with K long enough to cut: the tile kernel with K over several workgroups per tile as well (their
+		// tiles added through the scratch by the last to arrive), so that 32 to 191 column blocks still put a workgroup on
+		// every CU.  Measured against the streaming kernel: [8192 x 28672] M = 64 / 32 / 16: 52 / 46 / 46 against 70 / 52 / 48
+		// us; [8192 x 8192]: 23.7 / 18.0 / 17.6 against 24.1 / 19.0 / 18.4; [14336 x 4096] M = 64: 20.5 against 22.9 (M = 32:
+		// 16.8 against 16.2, left where it was); [4096 x 14336] M = 64: 24.0 against 26.2 (M = 16: 19.8 against 18.0);
+		// [1024 x 8192] M = 64: 13.5 against 11.7.
+		if (!sums && M <= GEMM_SKINNY_MAX_M && (M > 32 ? column_blocks >= 32 : (M >= 16 && column_blocks >= 64 && K >= 8192))) {
+			return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, true);
+		}
 		if (M <= GEMM_SKINNY_MAX_M && column_blocks >= GEMM_STREAM_TILE_MIN_COLUMN_BLOCKS) {
 			return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, true);
 		}

@@ -254,6 +254,7 @@ __global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kerne
 // Scratch of the K-split path (partial 32x32 tiles and arrival counters): one allocation per device on first use.
 constexpr int SK_MAX_SPLIT_UNITS  = 2048; // strips * splits when splits > 1
 constexpr int SK_MAX_SPLIT_STRIPS = 512;
+static_assert(GEMM_SPLIT_SCRATCH_FLOATS == SK_MAX_SPLIT_UNITS * 2 * 16 * 64 && GEMM_SPLIT_MAX_UNITS == SK_MAX_SPLIT_STRIPS, "one scratch, two users");
 struct skinny_scratch {
 	float* partials	   = nullptr;
 	unsigned* counters = nullptr;
@@ -306,6 +307,19 @@ static hipError_t get_skinny_scratch(skinny_scratch* out, bool launching = false
 		sc.has_user = true;
 	}
 	*out = sc;
+	return hipSuccess;
+}
+
+// The same scratch for the tile kernel's K split over workgroups (GEMM_SPLIT_SCRATCH_FLOATS floats of tiles, GEMM_SPLIT_MAX_UNITS
+// counters that every launch leaves at zero); same one-stream rule.
+hipError_t acquire_gemm_split_scratch(float** partials, unsigned** counters, hipStream_t s) {
+	skinny_scratch sc;
+	const hipError_t e = get_skinny_scratch(&sc, true, s);
+	if (e != hipSuccess) {
+		return e;
+	}
+	*partials = sc.partials;
+	*counters = sc.counters;
 	return hipSuccess;
 }
 
