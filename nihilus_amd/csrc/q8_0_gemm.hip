@@ -550,9 +550,9 @@ template<int TM, bool STREAM> static hipError_t launch_gemm_tiled_t(const uint8_
 	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 1, STREAM>, grid, dim3(256), 0, s, w, a, C, R, sums, m, n, groups, static_cast<float*>(nullptr), static_cast<unsigned*>(nullptr));
 }
 
-// Two activation strips per wave whenever there are two: every weight tile fetched is used twice, which halves what a CU
-// has to take in per MFMA (that intake, not the MFMA rate, bounds the one-strip form); the K sets give back the waves the
-// halved grid loses.  stream: the weights are read once and not again (a batch of decode rows against a large matrix), so
+// Two activation strips per wave whenever there are two: every weight tile fetched is used twice (the one-strip form,
+// with twice the weight loads per MFMA, measured 8 to 60 % slower at M = 512); the K sets give back the waves the halved
+// grid loses.  stream: the weights are read once and not again (a batch of decode rows against a large matrix), so
 // their loads bypass the caches.
 static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s, bool stream) {
 	const int64_t ms = (m + 31) / 32;
@@ -592,9 +592,9 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 		const int64_t tile_workgroups = column_blocks * ((M + 31) / 32);
 		// A matrix with enough 128-row column blocks to occupy the chip by itself takes the tile kernel at any M: its four
 		// waves share each activation tile through LDS, where the streaming kernel's eight waves fetch one each from L2 --
-		// at 32 to 64 rows that is one to two times the weight bytes in extra traffic into every CU, and what a CU can take
-		// in is what bounds both kernels ([28672 x 8192] at M = 16 / 32 / 64: 50 / 55 / 75 us streaming, 44 / 44 / 69 us
-		// here; [128256 x 8192]: 193 / - / 298 against 182 / - / 221 us).  Below that the tile kernel's grid leaves CUs idle
+		// at 32 to 64 rows that is one to two times the weight bytes in extra traffic into every CU ([28672 x 8192] at
+		// M = 16 / 32 / 64: 50 / 55 / 75 us streaming, 44 / 44 / 69 us here; [128256 x 8192]: 193 / - / 298 against
+		// 182 / - / 221 us).  Below that the tile kernel's grid leaves CUs idle
 		// ([14336 x 4096] at M = 64: 30 us against 23 us) and the streaming kernel, which can split K over workgroups, stays.
 		// Between the two, with K long enough to cut: the tile kernel with K over several workgroups per tile as well (their
 		// tiles added through the scratch by the last to arrive), so that 32 to 191 column blocks still put a workgroup on
