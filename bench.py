@@ -521,8 +521,13 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                     it[0] += 1
                     _lib.check("nh_q8_0_mul_mat", lib.nh_q8_0_mul_mat(w.data_ptr(), xm.data_ptr(), c.data_ptr(), m, n, k, wsp.data_ptr(), ws_bytes, stream))
 
-                for _ in range(warmup):
+                # from 16 rows on the MFMA kernels take these shapes and the shader clock has to settle first (see timed() above)
+                settle, t_warm, done = (0.15 if m >= 16 else 0.0), time.perf_counter(), 0
+                while done < warmup or time.perf_counter() - t_warm < settle:
                     fn()
+                    done += 1
+                    if done % 64 == 0:
+                        torch.cuda.synchronize()
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for _ in range(steps):
