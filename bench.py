@@ -408,11 +408,10 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
     steps = min(steps, 200)
     warmup = min(warmup, 20)
 
-    def timed(kind_id: int, fn, launches_per_step: int):
-        # The matrix kernel's time depends on the shader clock, and the clock needs ~0.1 s of sustained matrix work to settle after
-        # idling (a launch among the first few hundred reads up to 10 % slower than the same launch later): the mat-mat leg
-        # keeps warming up until 0.2 s have passed.  The bandwidth-bound kernels show no such dependence.
-        settle = 0.2 if kind == "prefill" else 0.0
+    def warm_up(fn, settle: float):
+        # The matrix kernels' time depends on the shader clock, and the clock needs ~0.1 s of sustained matrix work to settle after
+        # idling (a launch among the first few hundred reads up to 10 % slower than the same launch later): legs that run them
+        # keep warming up until `settle` seconds have passed.  The bandwidth-bound kernels show no such dependence.
         t_warm, done = time.perf_counter(), 0
         while done < warmup or time.perf_counter() - t_warm < settle:
             fn()
@@ -420,6 +419,9 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
             if done % 64 == 0:
                 torch.cuda.synchronize()
         torch.cuda.synchronize()
+
+    def timed(kind_id: int, fn, launches_per_step: int):
+        warm_up(fn, 0.2 if kind == "prefill" else 0.0)
         t0 = time.perf_counter()
         for _ in range(steps):
             fn()
@@ -480,9 +482,7 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                 def fn():
                     _lib.check("nh_q8_0_mul_mat", lib.nh_q8_0_mul_mat(w.data_ptr(), xm.data_ptr(), c.data_ptr(), m, n, k, wsp.data_ptr(), ws_bytes, stream))
 
-                for _ in range(warmup):
-                    fn()
-                torch.cuda.synchronize()
+                warm_up(fn, 0.15 if m >= 16 else 0.0)
                 t0 = time.perf_counter()
                 for _ in range(steps):
                     fn()
@@ -521,14 +521,7 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                     it[0] += 1
                     _lib.check("nh_q8_0_mul_mat", lib.nh_q8_0_mul_mat(w.data_ptr(), xm.data_ptr(), c.data_ptr(), m, n, k, wsp.data_ptr(), ws_bytes, stream))
 
-                # from 16 rows on the MFMA kernels take these shapes and the shader clock has to settle first (see timed() above)
-                settle, t_warm, done = (0.15 if m >= 16 else 0.0), time.perf_counter(), 0
-                while done < warmup or time.perf_counter() - t_warm < settle:
-                    fn()
-                    done += 1
-                    if done % 64 == 0:
-                        torch.cuda.synchronize()
-                torch.cuda.synchronize()
+                warm_up(fn, 0.15 if m >= 16 else 0.0)  # from 16 rows on the MFMA kernels take these shapes
                 t0 = time.perf_counter()
                 for _ in range(steps):
                     fn()

@@ -601,8 +601,10 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 		// every CU.  Measured against the streaming kernel: [8192 x 28672] M = 64 / 32 / 16: 52 / 46 / 46 against 70 / 52 / 48
 		// us; [8192 x 8192]: 23.7 / 18.0 / 17.6 against 24.1 / 19.0 / 18.4; [14336 x 4096] M = 64: 20.5 against 22.9 (M = 32:
 		// 16.8 against 16.2, left where it was); [4096 x 14336] M = 64: 24.0 against 26.2 (M = 16: 19.8 against 18.0);
-		// [1024 x 8192] M = 64: 13.5 against 11.7.
-		if (!sums && M <= GEMM_SKINNY_MAX_M && (M > 32 ? column_blocks >= 32 : (M >= 16 && column_blocks >= 64 && K >= 8192))) {
+		// [1024 x 8192] M = 64: 13.5 against 11.7;
+		// [4096 x 4096] M = 64: 13.6 against 10.3.  So: two row strips from 48 Mi weights on, one (16 rows or more) from 64 Mi.
+		const int64_t weights = N * K;
+		if (!sums && M <= GEMM_SKINNY_MAX_M && (M > 32 ? (column_blocks >= 32 && weights >= (48ll << 20)) : (M >= 16 && column_blocks >= 64 && weights >= (64ll << 20)))) {
 			return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, true);
 		}
 		if (M <= GEMM_SKINNY_MAX_M && column_blocks >= GEMM_STREAM_TILE_MIN_COLUMN_BLOCKS) {
