@@ -4,9 +4,11 @@ from __future__ import annotations
 import os
 import shutil
 import subprocess
+from concurrent.futures import ThreadPoolExecutor
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
+OBJ_DIR = os.path.join(CSRC, "build")
 LIB_NAME = "libnihilus_q8_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
@@ -19,7 +21,6 @@ HIPCC_FLAGS = [
     "-O3",
     "-std=c++20",
     "-fPIC",
-    "-shared",
     "-fno-fast-math",
     "-ffp-contract=off",
     "-Wall",
@@ -29,6 +30,8 @@ HIPCC_FLAGS = [
     # result parked in an accumulation register would cost one extra copy instruction per value (doubling the VALU work)
     "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
+# the host pass does not know the packed-fp32 feature name and says so once per source: not an error
+NOISE = "is not a recognized feature for this target"
 
 
 def hipcc() -> str:
@@ -38,20 +41,52 @@ def hipcc() -> str:
     return exe
 
 
-def build_library(verbose: bool = False, extra_flags: list[str] | None = None) -> str:
-    """Compile every HIP source into one shared library next to this file. Always recompiles."""
-    include = os.path.join(os.path.dirname(PKG_DIR), "include")
-    cmd = [hipcc(), *HIPCC_FLAGS, "-I", include, *(extra_flags or []), "-o", LIB_PATH, *[os.path.join(CSRC, s) for s in SOURCES]]
+def _run(cmd: list[str]) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
-    # the host pass does not know the packed-fp32 feature name and says so once per source: not an error
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    err = "\n".join(l for l in res.stderr.splitlines() if NOISE not in l)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{' '.join(cmd)}\n{err}")
-    if verbose and err.strip():
-        print(err)
+    return err
+
+
+def _newest_header_mtime(include: str) -> float:
+    newest = 0.0
+    for folder in (CSRC, os.path.join(include, "nihilus_amd")):
+        for name in os.listdir(folder):
+            if name.endswith(".h"):
+                newest = max(newest, os.path.getmtime(os.path.join(folder, name)))
+    return newest
+
+
+def build_library(verbose: bool = False, extra_flags: list[str] | None = None, incremental: bool = False, jobs: int = 8) -> str:
+    """Compile every HIP source to an object (in parallel) and link them into one shared library next to this file.
+
+    Recompiles everything unless incremental=True, which keeps objects newer than their source and every header.
+    """
+    include = os.path.join(os.path.dirname(PKG_DIR), "include")
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    flags = [*HIPCC_FLAGS, "-I", include, *(extra_flags or [])]
+    headers = _newest_header_mtime(include)
+
+    def compile_one(src: str) -> str:
+        path = os.path.join(CSRC, src)
+        obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+        if incremental and not extra_flags and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(path), headers):
+            return ""
+        return _run([hipcc(), *flags, "-c", path, "-o", obj])
+
+    with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        notes = list(pool.map(compile_one, SOURCES))
+    objs = [os.path.join(OBJ_DIR, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+    notes.append(_run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]))
+    if verbose:
+        text = "\n".join(n for n in notes if n.strip())
+        if text:
+            print(text)
     return LIB_PATH
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    import sys
+
+    print(build_library(verbose=True, incremental="--incremental" in sys.argv))
