@@ -22,7 +22,10 @@
 // kernels); prompt_eval_time bodies quantize into a workspace and run the int8-MFMA mat-mat.
 //
 // What those cores hold besides mat-muls is outside this path and is reached through three customisation points that a
-// config specialises (the primary templates below do the minimum that keeps the data flowing):
+// config MUST specialise: without them a model runs and produces garbage (no rope, no cache write, q standing in for the
+// attention output, no sampled token).  The primary templates therefore refuse to compile, unless the config declares
+// `static constexpr bool amd_matmul_only = true` -- what a benchmark or a test of the mat-mul path alone does -- in which case
+// they do the minimum that keeps the data flowing:
 //   amd_qkv_epilogue<config>    rope on q and k, the k / v cache write              (reshape/rope/copy nodes, core_traits.hpp:596-616)
 //   amd_attention<config>       k.q, softmax, .v, merge: produces the attn_out operand  (core_traits.hpp:743-766)
 //   amd_sampling<config>        logit bias, penalties, top-k/p, sample               (core_traits.hpp:1195-1227)
@@ -46,27 +49,48 @@ namespace nihilus {
 
 		// Device memory the bodies need beyond the graph's own tensors: quantized activations of the prompt phase, the k / v
 		// projections in front of the cache write, the fp32 gate / up outputs of a prompt-phase FFN, the logits.  The
-		// reference's memory planner sizes its arena from the graph nodes alone (infra/core_traits.hpp:130-141), so these
-		// live in a per-process pool of grow-only slots: the first call of a shape allocates, later calls of that or a
-		// smaller shape allocate nothing.  One host thread drives the GPU (cuda/thread_pool.hpp:46-67).
+		// reference's kernels never allocate: its arena is sized once from a compile-time plan over the graph nodes
+		// (infra/behavioral_axes.hpp:61-90, infra/model.hpp:241).  Here the same happens in amd_prepare (below): every slot is
+		// sized once for the longest sequence the config allows, and the dispatchers only check capacity.  One host thread
+		// drives the GPU (cuda/thread_pool.hpp:46-67).
 		enum workspace_slot : int { slot_quantized = 0, slot_k, slot_v, slot_gate, slot_up, slot_attention, slot_logits, slot_count };
+		struct workspace_entry {
+			void* ptr{};
+			int64_t bytes{};
+		};
+		template<typename config_type> struct workspace_pool {
+			workspace_entry slots[slot_count]{};
+			std::mutex lock{};
+			int64_t allocations{}; // nh_malloc calls made for this config so far (a test reads it: none after amd_prepare)
+			static workspace_pool& get() {
+				static workspace_pool pool{};
+				return pool;
+			}
+		};
+		// A slot of at least `bytes`.  Allocates nothing: a slot that amd_prepare did not make large enough is an error.
 		template<typename config_type> inline void* workspace(int slot, int64_t bytes, const std::source_location where = std::source_location::current()) {
-			struct entry {
-				void* ptr{};
-				int64_t bytes{};
-			};
-			static entry slots[slot_count];
-			static std::mutex lock;
-			std::lock_guard<std::mutex> guard{ lock };
-			entry& e = slots[slot];
+			auto& pool = workspace_pool<config_type>::get();
+			std::lock_guard<std::mutex> guard{ pool.lock };
+			const workspace_entry& e = pool.slots[slot];
 			if (e.bytes < bytes) {
-				check<config_type>(nh_stream_sync(nullptr), "workspace: stream sync", where); // the old buffer may still be in use by enqueued work
-				check<config_type>(nh_free(e.ptr), "workspace: free", where);
-				e = entry{};
-				check<config_type>(nh_malloc(&e.ptr, (bytes + 255) / 256 * 256), "workspace: alloc", where);
-				e.bytes = (bytes + 255) / 256 * 256;
+				check<config_type>(NH_ERR_TOO_LARGE, "workspace: call nihilus::amd_prepare<config, model_traits>(max_sequence_length) first, with a sequence length that covers this call", where);
+				return nullptr;
 			}
 			return e.ptr;
+		}
+		template<typename config_type> inline void reserve_slot(int slot, int64_t bytes, const std::source_location where = std::source_location::current()) {
+			auto& pool = workspace_pool<config_type>::get();
+			std::lock_guard<std::mutex> guard{ pool.lock };
+			workspace_entry& e = pool.slots[slot];
+			bytes			   = (bytes + 255) / 256 * 256;
+			if (e.bytes < bytes) {
+				check<config_type>(nh_stream_sync(nullptr), "amd_prepare: stream sync", where); // the old buffer may still be in use by enqueued work
+				check<config_type>(nh_free(e.ptr), "amd_prepare: free", where);
+				e = workspace_entry{};
+				check<config_type>(nh_malloc(&e.ptr, bytes), "amd_prepare: alloc", where);
+				e.bytes = bytes;
+				++pool.allocations;
+			}
 		}
 
 		// get_data() of a graph node, per transformer block or global as the node's data strategy says.
@@ -86,6 +110,15 @@ namespace nihilus {
 			}
 		}
 
+		// A config that runs the mat-mul path alone (benchmarks, tests) says so; only then do the primary customisation points compile.
+		template<typename config_type> inline constexpr bool matmul_only = [] {
+			if constexpr (requires { config_type::amd_matmul_only; }) {
+				return static_cast<bool>(config_type::amd_matmul_only);
+			} else {
+				return false;
+			}
+		}();
+
 		// The input of transformer block `current_block`: token embeddings for the first, the previous block's l_out afterwards.
 		template<typename core_traits_type> inline const float* layer_input(core_traits_type& params, int64_t current_block) {
 			using config_type = typename core_traits_type::config_type;
@@ -99,31 +132,69 @@ namespace nihilus {
 
 	} // namespace amd_detail
 
+	// ---- set-up ---------------------------------------------------------------------------------------------------------
+
+	// Sizes every device buffer the dispatchers below need beyond the graph's tensors, once, for sequences of up to
+	// `max_sequence_length` rows, and has the library make its own per-device scratch (nh_q8_0_prepare).  Call it after the
+	// model's memory is set up and before the first impl: from then on no impl allocates, frees or waits for the device on
+	// behalf of memory (a sequence longer than prepared for is reported through the config's error convention).  Stands for
+	// the reference's compile-time memory plan (infra/behavioral_axes.hpp:61-90).  model_traits_type: the mtt of the config's
+	// core traits (embedding_length, feed_forward_length, n_embd_kv_gqa, vocab_size).
+	template<typename config_type, typename model_traits_type> inline void amd_prepare(uint64_t max_sequence_length = config_type::max_sequence_length) {
+		const int64_t rows	 = max_sequence_length < 1 ? 1 : static_cast<int64_t>(max_sequence_length);
+		const int64_t n_embd = model_traits_type::embedding_length, n_ff = model_traits_type::feed_forward_length, n_kv = model_traits_type::n_embd_kv_gqa;
+		int64_t quantized	 = nh_q8_0_tiled_bytes(rows, n_embd);
+		for (const int64_t other : { nh_q8_0_tiled_bytes(rows, n_ff), nh_q8_0_mul_mat_workspace_bytes(rows, n_embd), nh_q8_0_mul_mat_workspace_bytes(rows, n_ff) }) {
+			quantized = other > quantized ? other : quantized;
+		}
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_quantized, quantized);
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_k, rows * n_kv * 4);
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_v, rows * n_kv * 4);
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_gate, rows * n_ff * 4);
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_up, rows * n_ff * 4);
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_attention, rows * n_embd * 4);
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_logits, static_cast<int64_t>(model_traits_type::vocab_size) * 4);
+		amd_detail::check<config_type>(nh_q8_0_prepare(), "amd_prepare: library scratch");
+	}
+	// How many device allocations amd_prepare has made for this config (a later amd_prepare with a longer sequence adds to it; impl never does).
+	template<typename config_type> inline int64_t amd_workspace_allocations() {
+		auto& pool = amd_detail::workspace_pool<config_type>::get();
+		std::lock_guard<std::mutex> guard{ pool.lock };
+		return pool.allocations;
+	}
+
 	// ---- customisation points for the nodes of a mega core that are not mat-muls --------------------------------------
 
 	// After the q / k / v projections: q [sequence_length][embedding_length] sits in the core's q_out tensor, k and v
 	// [sequence_length][n_embd_kv_gqa] in scratch.  A config's specialisation applies rope to q and k and writes k / v into
-	// the cache (params.data_ptrs holds inp_pos, rope_freqs, cache_k, cache_v).  Primary: nothing.
+	// the cache (params.data_ptrs holds inp_pos, rope_freqs, cache_k, cache_v).  Primary (amd_matmul_only configs): nothing.
 	template<typename config_type> struct amd_qkv_epilogue {
 		template<typename core_traits_type>
 		static void impl(core_traits_type&, int64_t /*current_block*/, uint64_t /*sequence_length*/, float* /*q*/, const float* /*k*/, const float* /*v*/, void* /*stream*/) {
+			static_assert(amd_detail::matmul_only<config_type>,
+				"specialise nihilus::amd_qkv_epilogue<config> (rope on q and k, k / v cache write), or declare config::amd_matmul_only = true to run the mat-mul path alone");
 		}
 	};
 
 	// In front of the attn_out projection: returns the attention output, fp32 [sequence_length][embedding_length].  A config's
-	// specialisation runs k.q, softmax, .v and the head merge into `scratch` and returns it.  Primary: the q tensor itself
-	// (attention over a single cached position with v = q), which keeps shapes and data flow those of the model.
+	// specialisation runs k.q, softmax, .v and the head merge into `scratch` and returns it.  Primary (amd_matmul_only configs):
+	// the q tensor itself (attention over a single cached position with v = q), which keeps shapes and data flow those of the model.
 	template<typename config_type> struct amd_attention {
 		template<typename core_traits_type>
 		static const float* impl(core_traits_type& params, int64_t /*current_block*/, uint64_t /*sequence_length*/, float* /*scratch*/, void* /*stream*/) {
+			static_assert(amd_detail::matmul_only<config_type>,
+				"specialise nihilus::amd_attention<config> (k.q, softmax, .v, head merge), or declare config::amd_matmul_only = true to run the mat-mul path alone");
 			return params.data_ptrs.template get_q_input_data<float>();
 		}
 	};
 
 	// Behind the logits mat-vec: logits fp32 [vocab_size] of the last token.  A config's specialisation applies the sampling
-	// chain and writes params.data_ptrs.get_result_token_id_data.  Primary: nothing (the logits stay in the scratch slot).
+	// chain and writes params.data_ptrs.get_result_token_id_data, which the reference's generation loop reads next.  Primary
+	// (amd_matmul_only configs): nothing (the logits stay in the scratch slot, no token id is written).
 	template<typename config_type> struct amd_sampling {
 		template<typename core_traits_type> static void impl(core_traits_type&, const float* /*logits*/, void* /*stream*/) {
+			static_assert(amd_detail::matmul_only<config_type>,
+				"specialise nihilus::amd_sampling<config> (sampling chain, writes result_token_id), or declare config::amd_matmul_only = true to run the mat-mul path alone");
 		}
 	};
 

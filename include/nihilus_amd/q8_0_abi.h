@@ -26,7 +26,8 @@
  *   The check queries the other stream; it does so in the relaxed capture mode, so it may run while a third stream of the
  *   calling thread is being captured in the global mode without disturbing that capture.
  *   A kernel that waits for another workgroup's data does so for a bounded time; if it gives up, the output holds NaN and
- *   the next nh_stream_sync (or nh_q8_0_last_error) on that GPU returns NH_ERR_DEVICE_TIMEOUT once.
+ *   every nh_stream_sync and nh_q8_0_last_error on that GPU returns NH_ERR_DEVICE_TIMEOUT from then on, whichever stream or
+ *   thread asks, until nh_q8_0_clear_error resets it (one word per GPU: it says that some launch failed, not which).
  *
  * Data layouts
  *   "blocks"  the reference's wire layout: rows of packed 34-byte block_q8_0 { fp16 d; int8 qs[32] }
@@ -87,11 +88,15 @@ int nh_memcpy_d2h(void* host_dst, const void* src_dev, int64_t bytes, void* stre
  * point of this library clears memory with fill kernels instead and can be captured). */
 int nh_memset(void* dst_dev, int value, int64_t bytes, void* stream);
 /* Blocks until the stream has drained: the cudaDeviceSynchronize after each launch in cuda/cuda_12.hpp:679.  Returns
- * NH_ERR_DEVICE_TIMEOUT (once) if a kernel on this GPU gave up a bounded wait since the last report. */
+ * NH_ERR_DEVICE_TIMEOUT if a kernel on this GPU has given up a bounded wait since the last nh_q8_0_clear_error. */
 int nh_stream_sync(void* stream);
-/* Reads and clears the GPU's sticky device-side error without waiting for anything: NH_OK or NH_ERR_DEVICE_TIMEOUT.  The
- * reference looks at the device's error state after a launch only in dev builds (cuda/cuda_12.hpp:650-655). */
+/* The GPU's sticky device-side error, read without waiting for anything and without resetting it: NH_OK or
+ * NH_ERR_DEVICE_TIMEOUT.  The reference looks at the device's error state after a launch only in dev builds
+ * (cuda/cuda_12.hpp:650-655). */
 int nh_q8_0_last_error(void);
+/* Resets that error and returns what it held (NH_OK or NH_ERR_DEVICE_TIMEOUT): for the owner of the failed launch, once it has
+ * dealt with the NaN output.  A sync of an unrelated stream never resets it. */
+int nh_q8_0_clear_error(void);
 /* Allocates, for the current device, the two internal scratch buffers that K-split launches hand partial sums through
  * (about 2.6 MiB and 16 MiB; otherwise made by the first launch that needs one).  After it no launch entry point of this library
  * allocates device memory: call it once per device before capturing launches into a HIP graph or entering a serving loop.
@@ -171,8 +176,9 @@ int nh_q8_0_gemv_tiled_residual_f32(const void* W_tiled, const float* x, const f
  * the process ends) instead of a buffer allocated on first use.  The call allocates and frees nothing.  A shape whose cut
  * needs more than NH_Q8_0_NOALLOC_MAX_SPLIT_UNITS (32-row strip, K part) slots is rejected with NH_ERR_TOO_LARGE before
  * anything is launched ([4096 x 14336] uses 512, [8192 x 28672] 2048; shapes that need no K split always fit).  Every call on
- * a GPU shares that GPU's array: two such calls must not overlap on one GPU (run them on one stream).  No counterpart in the
- * reference, whose kernels never allocate (infra/model.hpp:241 owns the arena). */
+ * a GPU shares that GPU's array: two such calls must not overlap on one GPU (run them on one stream; a call on another stream
+ * while the previous user's stream still has work in flight returns NH_ERR_BUSY and launches nothing, as described under
+ * "Streams").  No counterpart in the reference, whose kernels never allocate (infra/model.hpp:241 owns the arena). */
 #define NH_Q8_0_NOALLOC_MAX_SPLIT_UNITS 2048
 int nh_q8_0_gemv_tiled_f32_noalloc(const void* W_tiled, const float* x, float* y, int64_t N, int64_t K, void* stream);
 /* The same for up to 3 weight matrices that share K and x (q/k/v, gate/up: infra/core_traits.hpp:575-594, :976-986)
@@ -294,9 +300,24 @@ int nh_q8_0_debug_fused_norm_quantize(const float* x, const float* norm_weight, 
  * library otherwise), copied out for comparison. */
 int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void* stream);
 
+/* Which kernel nh_q8_0_mul_mat(M, N, K) runs and how that kernel cuts the work: the launchers execute exactly this plan, so a
+ * test can pin the route of a shape (and a parity test can assert that the variant it means to cover is the one that runs).
+ * Needs no GPU.  host_plan receives eight int32:
+ *   [0] kernel: 0 nothing (empty problem), 1 fused quantize + streaming mat-vec (M == 1), 2 the same kernel with one dot product
+ *       per row (a few rows), 3 weight-streaming MFMA kernel, 4 MFMA tile kernel with non-temporal weights (batched decode on
+ *       large matrices), 5 MFMA tile kernel (prefill);
+ *   [1] 1 when the activations are quantized by a launch of their own into the workspace (kernels 3, 4, 5);
+ *   kernel 1:    [2] workgroups per 32-row strip along K, [3] 128-quant groups per wave, [4] row parts per strip;
+ *   kernel 3:    [2] 32-row activation strips per workgroup, [3] workgroups per weight strip along K;
+ *   kernel 4, 5: [2] activation strips per wave, [3] K sets of four waves per workgroup, [4] workgroups per tile along K,
+ *                [5], [6] the grid (column blocks of 128 weight rows, groups of activation strips);
+ *   the rest 0.  The same shape under HIP graph capture may take a form without state between launches (no K split). */
+int nh_q8_0_debug_plan_mul_mat(int64_t M, int64_t N, int64_t K, int32_t* host_plan);
+
 /* How many polls a workgroup of nh_q8_0_ffn_f32 waits for another workgroup's data before it gives up (default and upper
  * limit 2^20, lower limit 1).  Test hook for the time-out report: with a limit of 1 the down projection's workgroups find
- * their activation missing and give up while every kernel still runs to its end.  Process-wide. */
+ * their activation missing and give up while every kernel still runs to its end.  Process-wide, and refused with
+ * NH_ERR_ARGUMENT unless the process was started with NH_Q8_0_DEBUG_HOOKS=1 in its environment. */
 int nh_q8_0_debug_set_spin_limit(int64_t polls);
 
 /* Synthetic inputs (benchmark / test utility) --------------------------------------------------- */

@@ -2,8 +2,9 @@
 // Nothing here computes; every rejected argument returns a negative nh_status before any launch, so a
 // malformed call can never reach a kernel with shapes the kernel does not expect.
 #include "../../include/nihilus_amd/q8_0_abi.h"
-#include "q8_0_gemv_tiled.h"
+#include "q8_0_plan.h"
 
+#include <cstdlib>
 #include <cstring>
 
 namespace {
@@ -189,15 +190,23 @@ int nh_memset(void* dst_dev, int value, int64_t bytes, void* stream) {
 int nh_stream_sync(void* stream) {
 	NH_TRY(require_device());
 	NH_TRY(from_hip(hipStreamSynchronize(as_stream(stream))));
-	return nh::take_device_error() != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
+	return nh::read_device_error(false) != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
 }
 
 int nh_q8_0_last_error(void) {
 	NH_TRY(require_device());
-	return nh::take_device_error() != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
+	return nh::read_device_error(false) != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
+}
+
+int nh_q8_0_clear_error(void) {
+	NH_TRY(require_device());
+	return nh::read_device_error(true) != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
 }
 
 int nh_q8_0_debug_set_spin_limit(int64_t polls) {
+	// a test hook in a production library: it only works for a process that asked for it
+	const char* hooks = std::getenv("NH_Q8_0_DEBUG_HOOKS");
+	NH_REQUIRE(hooks && hooks[0] == '1' && hooks[1] == '\0', NH_ERR_ARGUMENT);
 	NH_REQUIRE(polls >= 1, NH_ERR_ARGUMENT);
 	nh::set_published_spin_limit(polls > nh::PUBLISHED_SPIN_LIMIT ? nh::PUBLISHED_SPIN_LIMIT : static_cast<int>(polls));
 	return NH_OK;
@@ -574,10 +583,11 @@ static int mul_mat_common(const void* W_tiled, const float* x, const float* resi
 		NH_REQUIRE(x && (workspace || need == 0), NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(workspace) && aligned16(x), NH_ERR_ALIGNMENT);
 	}
+	const nh::mul_mat_plan plan = nh::plan_mul_mat(M, N, K); // which kernel: q8_0_plan.h
 	if (M == 1) { // quantize fused into the mat-vec: the workspace stays unused
 		return residual ? nh_q8_0_gemv_tiled_residual_f32(W_tiled, x, residual, y, N, K, stream) : nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream);
 	}
-	if (nh::gemv_rows_suits(M, N, K) && K > 0) { // a few rows: the same streaming kernel with M dot products per weight tile
+	if (plan.kernel == nh::MM_GEMV_ROWS) { // a few rows: the same streaming kernel with M dot products per weight tile
 		NH_REQUIRE(W_tiled && y, NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(W_tiled) && aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
 		NH_TRY(require_device());
@@ -585,6 +595,39 @@ static int mul_mat_common(const void* W_tiled, const float* x, const float* resi
 	}
 	NH_TRY(nh_q8_0_quantize_tiled(x, workspace, M, K, stream));
 	return residual ? nh_q8_0_gemm_tiled_residual(W_tiled, workspace, residual, y, M, N, K, stream) : nh_q8_0_gemm_tiled(W_tiled, workspace, y, M, N, K, stream);
+}
+
+int nh_q8_0_debug_plan_mul_mat(int64_t M, int64_t N, int64_t K, int32_t* host_plan) {
+	NH_TRY(check_shape(M, N, K, true));
+	NH_REQUIRE(host_plan, NH_ERR_NULL_POINTER);
+	const nh::mul_mat_plan p = nh::plan_mul_mat(M, N, K);
+	for (int i = 0; i < 8; ++i) {
+		host_plan[i] = 0;
+	}
+	host_plan[0] = p.kernel;
+	host_plan[1] = p.quantize_launch;
+	switch (p.kernel) {
+		case nh::MM_GEMV:
+			host_plan[2] = p.gemv.splits;
+			host_plan[3] = p.gemv.tiles;
+			host_plan[4] = p.gemv_row_parts;
+			break;
+		case nh::MM_GEMM_SKINNY:
+			host_plan[2] = p.gemm.skinny.ms;
+			host_plan[3] = p.gemm.skinny.splits;
+			break;
+		case nh::MM_GEMM_TILE_STREAM:
+		case nh::MM_GEMM_TILE:
+			host_plan[2] = p.gemm.tile.tm;
+			host_plan[3] = p.gemm.tile.ks;
+			host_plan[4] = p.gemm.tile.kz;
+			host_plan[5] = static_cast<int32_t>(p.gemm.tile.grid_x);
+			host_plan[6] = static_cast<int32_t>(p.gemm.tile.grid_y);
+			break;
+		default:
+			break;
+	}
+	return NH_OK;
 }
 
 int nh_q8_0_mul_mat(const void* W_tiled, const float* x, float* y, int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {

@@ -12,7 +12,7 @@
 // Operand lanes: lane l supplies row (l % 32), quants 16*(l/32)..+15 of the block -- the tiled layout stores
 // tiles in exactly that order, so operands go from memory to the MFMA with one 16-byte load per lane and no
 // shuffle.  Result lanes: register i of lane l is C[m = 8*(i/4) + 4*(l/32) + i%4][n = l % 32].
-#include "q8_0_device.h"
+#include "q8_0_plan.h"
 
 namespace nh {
 
@@ -23,8 +23,6 @@ constexpr int GEMM_TN	   = 2; // along N
 constexpr int GEMM_BM	   = GEMM_WAVES_M * GEMM_TM * 32; // 128
 constexpr int GEMM_BN	   = GEMM_WAVES_N * GEMM_TN * 32; // 128
 constexpr int GEMM_THREADS = GEMM_WAVES_M * GEMM_WAVES_N * 64;
-constexpr int GEMM_SPLIT_MIN_TRIPS = 2; // K goes over more workgroups only while each K set keeps this many 128-quant groups
-constexpr int GEMM_STREAM_TILE_MIN_COLUMN_BLOCKS = 192; // 128-row column blocks from which the tile kernel also takes the few-row (batched decode) shapes
 
 // 16 operand bytes for (row strip, block b): lane supplies row strip*32 + lane%32, half lane/32.
 template<bool TILED> __device__ __forceinline__ v4i load_operand(const uint8_t* base, int rows, int nb, int strip, int b, int lane) {
@@ -509,35 +507,25 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	}
 }
 
-template<int TM, bool STREAM> static hipError_t launch_gemm_tiled_t(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s) {
-	const int groups   = k / GROUP_K;
-	const int m_strips = (m + 31) / 32, n_strips = (n + 31) / 32;
-	const dim3 grid(static_cast<unsigned>((n_strips + 3) / 4), static_cast<unsigned>((m_strips + TM - 1) / TM));
+// Executes a cut made by plan_gemm_tile (q8_0_plan.h): TM activation strips per wave, KS sets of four waves per workgroup,
+// and, with non-temporal weights, K over kz workgroups per tile whose tiles are added through the scratch.
+template<int TM, bool STREAM> static hipError_t launch_gemm_tiled_t(const gemm_tile_cut& cut, const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s) {
+	const int groups = k / GROUP_K;
+	const dim3 grid(cut.grid_x, cut.grid_y);
 	if (sums) {
 		gemm_tiled_kernel<TM, true><<<grid, dim3(256), 0, s>>>(w, a, C, R, sums, m, n, groups, nullptr, nullptr);
 		return hipGetLastError();
 	}
-	// a grid that leaves SIMDs short of their four waves: K sets inside the workgroup (8 or 16 waves) make up for it
-	int ks = 1;
-	while (ks < 4 && static_cast<int64_t>(grid.x) * grid.y * 4 * ks * 2 <= 4096 && groups % (ks * 2) == 0 && groups / (ks * 2) >= 4) {
-		ks *= 2;
-	}
+	const int ks = cut.ks;
 	if constexpr (STREAM) {
-		// still short of one workgroup per CU: K over kz workgroups per tile as well, their tiles added through the scratch
-		const int64_t wgs = static_cast<int64_t>(grid.x) * grid.y;
-		int kz = 1;
-		while (ks == 4 && wgs * kz * 2 <= 256 && groups % (ks * kz * 2) == 0 && groups / (ks * kz * 2) >= GEMM_SPLIT_MIN_TRIPS && wgs * kz * 2 * TM * 4096 <= GEMM_SPLIT_SCRATCH_FLOATS &&
-			wgs <= GEMM_SPLIT_MAX_UNITS) {
-			kz *= 2;
-		}
-		if (kz > 1) {
+		if (cut.kz > 1) {
 			float* partials	   = nullptr;
 			unsigned* counters = nullptr;
 			const hipError_t e = acquire_gemm_split_scratch(&partials, &counters, s);
 			if (e != hipSuccess) {
 				return e;
 			}
-			return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4, true, true>, dim3(grid.x, grid.y, static_cast<unsigned>(kz)), dim3(1024), 0, s, w, a, C, R, sums, m, n, groups, partials,
+			return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 4, true, true>, dim3(grid.x, grid.y, static_cast<unsigned>(cut.kz)), dim3(1024), 0, s, w, a, C, R, sums, m, n, groups, partials,
 				counters);
 		}
 	}
@@ -550,16 +538,12 @@ template<int TM, bool STREAM> static hipError_t launch_gemm_tiled_t(const uint8_
 	return launch_kernel(KIND_GEMM, gemm_tiled_kernel<TM, false, 1, STREAM>, grid, dim3(256), 0, s, w, a, C, R, sums, m, n, groups, static_cast<float*>(nullptr), static_cast<unsigned*>(nullptr));
 }
 
-// Two activation strips per wave whenever there are two: every weight tile fetched is used twice (the one-strip form,
-// with twice the weight loads per MFMA, measured 8 to 60 % slower at M = 512); the K sets give back the waves the halved
-// grid loses.  stream: the weights are read once and not again (a batch of decode rows against a large matrix), so
-// their loads bypass the caches.
-static hipError_t launch_gemm_tiled(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s, bool stream) {
-	const int64_t ms = (m + 31) / 32;
+// stream: the weights are read once and not again (a batch of decode rows against a large matrix), so their loads bypass the caches.
+static hipError_t launch_gemm_tiled(const gemm_tile_cut& cut, const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int k, hipStream_t s, bool stream) {
 	if (stream) {
-		return ms >= 2 ? launch_gemm_tiled_t<2, true>(w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, true>(w, a, C, R, sums, m, n, k, s);
+		return cut.tm == 2 ? launch_gemm_tiled_t<2, true>(cut, w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, true>(cut, w, a, C, R, sums, m, n, k, s);
 	}
-	return ms >= 2 ? launch_gemm_tiled_t<2, false>(w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, false>(w, a, C, R, sums, m, n, k, s);
+	return cut.tm == 2 ? launch_gemm_tiled_t<2, false>(cut, w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, false>(cut, w, a, C, R, sums, m, n, k, s);
 }
 
 __global__ void zero_c_kernel(float* c, const float* src, int64_t n) {
@@ -584,36 +568,14 @@ hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, i
 	const uint8_t* a = static_cast<const uint8_t*>(Aq);
 	const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
 	if (tiled) {
-		// Few rows: the weights are read once and the kernel is HBM-bound.  Somewhat more rows than that, but so few
-		// 128-row x 32-row tiles that the tile kernel would leave most SIMDs with one wave or none (measured: it needs
-		// more than one workgroup per CU to pay): the same streaming kernel over groups of 64 rows, K split over the
-		// waves of a workgroup, the weights coming from cache after the first group.
-		const int64_t column_blocks	  = (N + 127) / 128;
-		const int64_t tile_workgroups = column_blocks * ((M + 31) / 32);
-		// A matrix with enough 128-row column blocks to occupy the chip by itself takes the tile kernel at any M: its four
-		// waves share each activation tile through LDS, where the streaming kernel's eight waves fetch one each from L2 --
-		// at 32 to 64 rows that is one to two times the weight bytes in extra traffic into every CU ([28672 x 8192] at
-		// M = 16 / 32 / 64: 50 / 55 / 75 us streaming, 44 / 44 / 69 us here; [128256 x 8192]: 193 / - / 298 against
-		// 182 / - / 221 us).  Below that the tile kernel's grid leaves CUs idle
-		// ([14336 x 4096] at M = 64: 30 us against 23 us) and the streaming kernel, which can split K over workgroups, stays.
-		// Between the two, with K long enough to cut: the tile kernel with K over several workgroups per tile as well (their
-		// tiles added through the scratch by the last to arrive), so that 32 to 191 column blocks still put a workgroup on
-		// every CU.  Measured against the streaming kernel: [8192 x 28672] M = 64 / 32 / 16: 52 / 46 / 46 against 70 / 52 / 48
-		// us; [8192 x 8192]: 23.7 / 18.0 / 17.6 against 24.1 / 19.0 / 18.4; [14336 x 4096] M = 64: 20.5 against 22.9 (M = 32:
-		// 16.8 against 16.2, left where it was); [4096 x 14336] M = 64: 24.0 against 26.2 (M = 16: 19.8 against 18.0);
-		// [1024 x 8192] M = 64: 13.5 against 11.7;
-		// [4096 x 4096] M = 64: 13.6 against 10.3.  So: two row strips from 48 Mi weights on, one (16 rows or more) from 64 Mi.
-		const int64_t weights = N * K;
-		if (!sums && M <= GEMM_SKINNY_MAX_M && (M > 32 ? (column_blocks >= 32 && weights >= (48ll << 20)) : (M >= 16 && column_blocks >= 64 && weights >= (64ll << 20)))) {
-			return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, true);
+		if (sums) { // the inspection variant runs on the plain tile kernel, whatever the shape
+			return launch_gemm_tiled(plan_gemm_tile(M, N, K, false), w, a, C, residual, sums, m, n, k, s, false);
 		}
-		if (M <= GEMM_SKINNY_MAX_M && column_blocks >= GEMM_STREAM_TILE_MIN_COLUMN_BLOCKS) {
-			return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, true);
-		}
-		if (M <= GEMM_SKINNY_MAX_M || tile_workgroups <= 256) {
+		const gemm_plan plan = plan_gemm(M, N, K); // which kernel and how it cuts the work: q8_0_plan.h
+		if (plan.kernel == MM_GEMM_SKINNY) {
 			return launch_gemm_skinny(W, Aq, C, sums, M, N, K, s, residual);
 		}
-		return launch_gemm_tiled(w, a, C, residual, sums, m, n, k, s, false);
+		return launch_gemm_tiled(plan.tile, w, a, C, residual, sums, m, n, k, s, plan.kernel == MM_GEMM_TILE_STREAM);
 	} else {
 		if (sums) {
 			gemm_kernel<false, true><<<grid, dim3(GEMM_THREADS), 0, s>>>(w, a, C, sums, m, n, k);

@@ -9,13 +9,12 @@
 // columns.  Scale products come from a v_mfma_f32_32x32x8_f16 on the blocks' fp16 scales (exact, same register layout),
 // then one convert + one multiply-add per value.  Same arithmetic as the prefill kernel (reference
 // vec_dot_q8_0_q8_0, cpu/avx_2.hpp:4534-4747; output [M][N], n fastest, cpu/avx_2.hpp:4934).
-#include "q8_0_device.h"
+#include "q8_0_plan.h"
 
 #include <mutex>
 
 namespace nh {
 
-constexpr int SK_WAVES = 8;
 typedef _Float16 sk_v4h __attribute__((ext_vector_type(4)));
 typedef float sk_v16f __attribute__((ext_vector_type(16)));
 
@@ -252,8 +251,6 @@ __global__ __launch_bounds__(SK_WAVES * 64, DUMP ? 2 : 4) void gemm_skinny_kerne
 }
 
 // Scratch of the K-split path (partial 32x32 tiles and arrival counters): one allocation per device on first use.
-constexpr int SK_MAX_SPLIT_UNITS  = 2048; // strips * splits when splits > 1
-constexpr int SK_MAX_SPLIT_STRIPS = 512;
 static_assert(GEMM_SPLIT_SCRATCH_FLOATS == SK_MAX_SPLIT_UNITS * 2 * 16 * 64 && GEMM_SPLIT_MAX_UNITS == SK_MAX_SPLIT_STRIPS, "one scratch, two users");
 struct skinny_scratch {
 	float* partials	   = nullptr;
@@ -328,21 +325,9 @@ hipError_t prepare_gemm_scratch() {
 	return get_skinny_scratch(&sc);
 }
 
-template<int MS> static hipError_t launch_skinny_t(const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int groups, hipStream_t s) {
+template<int MS> static hipError_t launch_skinny_t(int splits, const uint8_t* w, const uint8_t* a, float* C, const float* R, int32_t* sums, int m, int n, int groups, hipStream_t s) {
 	const int strips   = (n + STRIP_ROWS - 1) / STRIP_ROWS;
 	const int m_groups = ((m + STRIP_ROWS - 1) / STRIP_ROWS + MS - 1) / MS;
-	const int units	   = strips * m_groups;
-	int splits		   = 1;
-	// The hand-off between workgroups is expensive here (a partial tile of 16 values per lane and strip, an arrival counter,
-	// the last arriver reading every share): K goes over several workgroups only until every CU has one (and every wave
-	// keeps at least four groups), or when a wave would otherwise walk more than sixteen groups.  Measured on [8192 x 28672]
-	// at M = 16: 68 us with eight workgroups per strip, 51 us with two.
-	while (units * splits < 256 && groups >= 8 * SK_WAVES * splits && units * splits * 2 <= SK_MAX_SPLIT_UNITS && units <= SK_MAX_SPLIT_STRIPS) {
-		splits *= 2;
-	}
-	while (groups > 16 * SK_WAVES * splits && units * splits * 2 <= SK_MAX_SPLIT_UNITS && units <= SK_MAX_SPLIT_STRIPS) {
-		splits *= 2;
-	}
 	skinny_scratch sc;
 	if (splits > 1) {
 		const hipError_t e = get_skinny_scratch(&sc, true, s);
@@ -366,13 +351,11 @@ hipError_t launch_gemm_skinny(const void* W, const void* Aq, float* C, int32_t* 
 	const uint8_t* w = static_cast<const uint8_t*>(W);
 	const uint8_t* a = static_cast<const uint8_t*>(Aq);
 	const int groups = static_cast<int>(K / GROUP_K);
-	// Two activation strips per workgroup halve the weight traffic per row, but only pay once the grid fills the chip
-	// without them: 64 rows against 128 weight strips are better off as 256 workgroups of one strip each.
-	const int64_t strips = (N + STRIP_ROWS - 1) / STRIP_ROWS, m_strips = (M + STRIP_ROWS - 1) / STRIP_ROWS;
-	if (m_strips <= 1 || strips * ((m_strips + 1) / 2) < 256) {
-		return launch_skinny_t<1>(w, a, C, residual, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
+	const gemm_skinny_cut cut = plan_gemm_skinny(M, N, K); // activation strips per workgroup, workgroups per strip: q8_0_plan.h
+	if (cut.ms == 1) {
+		return launch_skinny_t<1>(cut.splits, w, a, C, residual, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
 	}
-	return launch_skinny_t<2>(w, a, C, residual, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
+	return launch_skinny_t<2>(cut.splits, w, a, C, residual, sums, static_cast<int>(M), static_cast<int>(N), groups, s);
 }
 
 } // namespace nh

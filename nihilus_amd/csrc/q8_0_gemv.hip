@@ -11,7 +11,7 @@
 //   gemv_tiled_kernel   the streaming kernel on the tiled layout -- the one the decode path runs.
 // In both, lane l accumulates row (l % 32), quants 16*(l/32).. of every block, so the loop needs no cross-lane
 // reduction; halves and waves are combined once through LDS in a fixed order (run-to-run bit-stable).
-#include "q8_0_gemv_tiled.h"
+#include "q8_0_plan.h"
 
 #include <mutex>
 
@@ -300,7 +300,7 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch, hipStream_t s) {
 	return hipSuccess;
 }
 
-unsigned take_device_error() {
+unsigned read_device_error(bool clear) {
 	int dev = 0;
 	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
 		(void)hipGetLastError();
@@ -311,7 +311,7 @@ unsigned take_device_error() {
 	if (!word) {
 		return DEVICE_ERROR_NONE;
 	}
-	return __atomic_exchange_n(word, static_cast<unsigned>(DEVICE_ERROR_NONE), __ATOMIC_RELAXED);
+	return clear ? __atomic_exchange_n(word, static_cast<unsigned>(DEVICE_ERROR_NONE), __ATOMIC_RELAXED) : __atomic_load_n(word, __ATOMIC_RELAXED);
 }
 
 void set_published_spin_limit(int limit) {
@@ -340,11 +340,15 @@ __global__ void clear_tags_kernel(uint64_t* __restrict__ p, int n) {
 
 // The array's device address and the next epoch, per device.  First use on a device (that device current): look the
 // address up, then set every tag to zero, the one value no launch uses as its epoch (a fill kernel, not a memset node).
-// Calls that overlap on one GPU share the array and race on it, like the calls that share the allocated scratch.
+// Calls that overlap on one GPU share the array and would race on it, like the calls that share the allocated scratch: the
+// same one-stream-at-a-time rule applies (hipErrorNotReady while the previous user's stream, a different one, has work in
+// flight; the query allocates nothing).
 static hipError_t get_noalloc_scratch(gemv_scratch* out, hipStream_t s) {
 	struct state {
 		uint64_t* ptr  = nullptr;
 		unsigned epoch = 0;
+		hipStream_t user = nullptr; // stream of the last launch that used the array
+		bool has_user	 = false;
 	};
 	static std::mutex lock;
 	static state per_device[64];
@@ -358,6 +362,16 @@ static hipError_t get_noalloc_scratch(gemv_scratch* out, hipStream_t s) {
 	}
 	std::lock_guard<std::mutex> g(lock);
 	state& st = per_device[dev];
+	if (!stream_is_capturing(s)) {
+		if (st.has_user && st.user != s && st.user != nullptr) {
+			e = stream_drained(st.user); // also covers the first use's tag clearing, which went to that stream
+			if (e != hipSuccess) {
+				return e;
+			}
+		}
+		st.user		= s;
+		st.has_user = true;
+	}
 	if (!st.ptr) {
 		void* p = nullptr;
 		e		= hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
@@ -486,10 +500,7 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 	}
 	const int tiles = p.tiles <= 1 ? 1 : (p.tiles <= 2 ? 2 : 4);
 	if (dump_mode == DUMP_NONE && p.splits == 1) {
-		// Fewer strips than CUs (the 4096-row projections have 128, k/v 32): cut every strip into row parts so that the
-		// launch reaches RS times as many CUs.  What a single CU takes in per microsecond is limited, so half a chip
-		// cannot stream at the full HBM rate however many loads it has in flight.
-		const int rs = p.strips * 2 <= 256 ? (p.strips * 4 <= 256 ? 4 : 2) : 1;
+		const int rs = plan_gemv_row_parts(p); // fewer strips than CUs: row parts per strip (q8_0_plan.h)
 		if (rs == 4) {
 			return x_is_f32 ? launch_gemv_tiled_rs<4, true>(tiles, p, seg, x, sc, norm_w, norm_eps, s) : launch_gemv_tiled_rs<4, false>(tiles, p, seg, x, sc, norm_w, norm_eps, s);
 		}

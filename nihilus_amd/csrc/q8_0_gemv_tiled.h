@@ -469,8 +469,8 @@ struct gemv_scratch {
 // The check is skipped for capturing streams and when the previous user was the null stream (which may not be queried while
 // another stream captures).
 hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch = false, hipStream_t s = nullptr);
-// Reads and clears the current device's error word (DEVICE_ERROR_NONE if no scratch exists yet).
-unsigned take_device_error();
+// Reads the current device's error word (DEVICE_ERROR_NONE if no scratch exists yet); clear = true also resets it.
+unsigned read_device_error(bool clear);
 void set_published_spin_limit(int limit);
 
 // How a tiled mat-vec launch is cut: `splits` workgroups per strip, each of 16 waves owning <= `tiles` groups.

@@ -38,6 +38,25 @@ def tiled_bytes(rows: int, k: int) -> int:
     return n
 
 
+KERNEL_NAMES = {0: "nothing", 1: "gemv", 2: "gemv_rows", 3: "gemm_skinny", 4: "gemm_tile_stream", 5: "gemm_tile"}
+
+
+def plan_mul_mat(m: int, n: int, k: int) -> dict:
+    """Which kernel mul_mat runs for fp32 activations [m, k] against a tiled weight [n, k], and its cut (no GPU needed)."""
+    import ctypes
+
+    raw = (ctypes.c_int32 * 8)()
+    _lib.check("nh_q8_0_debug_plan_mul_mat", _lib.lib().nh_q8_0_debug_plan_mul_mat(m, n, k, raw))
+    plan = {"kernel": KERNEL_NAMES[raw[0]], "quantize_launch": bool(raw[1])}
+    if raw[0] == 1:
+        plan.update(k_splits=raw[2], groups_per_wave=raw[3], row_parts=raw[4])
+    elif raw[0] == 3:
+        plan.update(activation_strips=raw[2], k_splits=raw[3])
+    elif raw[0] in (4, 5):
+        plan.update(activation_strips=raw[2], k_sets=raw[3], k_splits=raw[4], grid=(raw[5], raw[6]))
+    return plan
+
+
 def quantize_row_q8_0(x: torch.Tensor, tiled: bool = False) -> torch.Tensor:
     """x fp32 [M, K] (or [K]) -> uint8 blocks [M, K/32*34] (or the tiled byte stream)."""
     x = _dev(x, torch.float32, "x")

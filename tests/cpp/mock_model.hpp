@@ -47,6 +47,7 @@ namespace nihilus {
 		static constexpr bool exceptions{ true };
 		static constexpr bool dev{ false };
 		static constexpr uint64_t max_sequence_length{ 64 };
+		static constexpr bool amd_matmul_only{ true }; // the mat-mul path alone: the header's stand-in customisation points may be used
 		using model_traits_type = NH_MOCK_MODEL_TRAITS;
 	};
 

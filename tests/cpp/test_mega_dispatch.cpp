@@ -235,10 +235,31 @@ int main(int argc, char** argv) {
 	static_cast<attn_core&>(model).values.get_core<mega_attention_apply_types, mega_attention_apply_types::ffn_inp>().set_data(d_ffn_inp);
 	static_cast<ffn_core&>(model).values.get_core<mega_ffn_types, mega_ffn_types::l_out>().set_data(d_l_out);
 
+	// every buffer the dispatchers need is sized once, up front; from here on no impl may allocate
+	amd_prepare<mock_config, mtt>(MAX_ROWS);
+	const int64_t allocations_after_prepare = amd_workspace_allocations<mock_config>();
+	REQUIRE(allocations_after_prepare == 7);
+
 	// eval_time: one token (the first row of x0); prompt_eval_time: 37 rows through the outputs' runtime dim
 	const std::vector<float> x_one(x0.begin(), x0.begin() + E);
 	REQUIRE(run_phase<processing_phases::eval_time>(model, wq, wk, wv, wo, wg, wu, wd, w_out, attn_norm, ffn_norm, out_norm, x_one, 1, d_q, d_ffn_inp, d_l_out) == 0);
 	REQUIRE(run_phase<processing_phases::prompt_eval_time>(model, wq, wk, wv, wo, wg, wu, wd, w_out, attn_norm, ffn_norm, out_norm, x0, ROWS, d_q, d_ffn_inp, d_l_out) == 0);
+
+	// a long prompt after a short one, and nothing was allocated on the way; preparing again for the same length allocates nothing either
+	REQUIRE(amd_workspace_allocations<mock_config>() == allocations_after_prepare);
+	amd_prepare<mock_config, mtt>(MAX_ROWS);
+	REQUIRE(amd_workspace_allocations<mock_config>() == allocations_after_prepare);
+
+	// a sequence longer than prepared for is refused through the config's error convention, before anything is launched
+	static_cast<ffn_core&>(model).values.get_core<mega_ffn_types, mega_ffn_types::l_out>().get_seq_length_dim() = MAX_ROWS + 1;
+	bool refused = false;
+	try {
+		kernel_dispatcher<mock_config, processing_phases::prompt_eval_time, ffn_core>::impl(static_cast<ffn_core&>(model), 0);
+	} catch (const std::runtime_error& e) {
+		refused = std::strstr(e.what(), "amd_prepare") != nullptr;
+	}
+	REQUIRE(refused);
+	REQUIRE(amd_workspace_allocations<mock_config>() == allocations_after_prepare);
 
 	// an empty sequence launches nothing
 	static_cast<ffn_core&>(model).values.get_core<mega_ffn_types, mega_ffn_types::l_out>().get_seq_length_dim() = 0;

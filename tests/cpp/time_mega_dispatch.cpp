@@ -88,6 +88,7 @@ int main(int argc, char** argv) {
 	REQUIRE(make_weight(&w_out, 10000, V, E, staging) == 0 && make_norm(&on, 10001, E) == 0);
 	weights.values.get_core<weight_types, weight_types::output>().set_data(w_out);
 	weights.values.get_core<weight_types, weight_types::output_norm>().set_data(on);
+	amd_prepare<mock_config, mtt>(1); // decode only: one row
 
 	void *d_x0, *d_q, *d_ffn_inp, *d_l_out;
 	REQUIRE(nh_malloc(&d_x0, E * 4) == NH_OK && nh_malloc(&d_q, E * 4) == NH_OK && nh_malloc(&d_ffn_inp, E * 4) == NH_OK && nh_malloc(&d_l_out, E * 4) == NH_OK);

@@ -108,7 +108,15 @@ def test_fails_loudly_without_a_gpu():
     assert lib.nh_q8_0_last_error() == -4
     # the status plumbing of the device-side reports needs no device
     assert "another stream" in _lib.status_string(-10) and "bounded wait" in _lib.status_string(-11)
-    assert lib.nh_q8_0_debug_set_spin_limit(0) == -6 and lib.nh_q8_0_debug_set_spin_limit(1 << 20) == 0
+    # the spin-limit test hook works only for a process that opted in through its environment
+    os.environ.pop("NH_Q8_0_DEBUG_HOOKS", None)
+    assert lib.nh_q8_0_debug_set_spin_limit(1 << 20) == -6
+    os.environ["NH_Q8_0_DEBUG_HOOKS"] = "1"
+    try:
+        assert lib.nh_q8_0_debug_set_spin_limit(0) == -6 and lib.nh_q8_0_debug_set_spin_limit(1 << 20) == 0
+    finally:
+        os.environ.pop("NH_Q8_0_DEBUG_HOOKS", None)
+    assert lib.nh_q8_0_clear_error() == -4
     assert lib.nh_q8_0_quantize(0x1000, 0x2000, 1, 32, None) == -4
     with pytest.raises(_lib.Q8Error):
         _lib.check("nh_q8_0_quantize", lib.nh_q8_0_quantize(0x1000, 0x2000, 1, 32, None))
@@ -165,6 +173,18 @@ def test_cpp_live_dispatch_point_compiles_against_the_reference_declaration():
     # the mode switch is real: the headers must not pull the mirror in when the reference's names are already there
     text = open(os.path.join(ROOT, "include", "nihilus_amd", "mul_mat_dispatch.hpp")).read()
     assert re.search(r"#ifndef NIHILUS_AMD_WITH_REFERENCE_HEADERS\s+#include \"reference_mirror.hpp\"", text)
+
+
+def test_customisation_points_must_be_specialised_by_a_real_config():
+    # a config without rope / attention / sampling hooks that does not declare amd_matmul_only must be stopped by the compiler
+    from nihilus_amd.build import hipcc
+
+    cxx = os.path.join(os.path.dirname(hipcc()), "amdclang++")
+    src = os.path.join(ROOT, "tests", "cpp", "customisation_points_are_mandatory.cpp")
+    res = subprocess.run([cxx, "-std=c++23", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "tests", "cpp"), src], capture_output=True, text=True)
+    errors = [ln for ln in res.stderr.splitlines() if " error: " in ln]
+    assert res.returncode != 0 and len(errors) == 1, res.stderr
+    assert "specialise nihilus::amd_attention<config>" in errors[0] and "amd_matmul_only" in errors[0]
 
 
 @pytest.mark.gpu

@@ -21,6 +21,60 @@ def _both(lib, wt, x, n, k, stream):
     return to_host(y_ref), to_host(y_new)
 
 
+def test_no_alloc_mat_vec_allocates_nothing(q8):
+    # Free device memory must not move across a call whose K split needs the hand-off array.  A first call on a shape without
+    # a split gets the runtime's own first-launch set-up out of the way (code object, kernel-argument pool); run alone in a
+    # fresh process, no allocating entry point has been called before this point, so a hidden hipMalloc would show.
+    lib = q8._lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    n0, k0, n, k = 14336, 4096, 4096, 14336
+    w0 = torch.zeros(q8.tiled_bytes(n0, k0), dtype=torch.uint8, device="cuda")
+    w = torch.zeros(q8.tiled_bytes(n, k), dtype=torch.uint8, device="cuda")
+    x = torch.ones(max(k0, k), dtype=torch.float32, device="cuda")
+    y = torch.empty(max(n0, n), dtype=torch.float32, device="cuda")
+    assert lib.nh_q8_0_gemv_tiled_f32_noalloc(w0.data_ptr(), x.data_ptr(), y.data_ptr(), n0, k0, stream) == 0
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(2):
+        assert lib.nh_q8_0_gemv_tiled_f32_noalloc(w.data_ptr(), x.data_ptr(), y.data_ptr(), n, k, stream) == 0
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    assert bool((y[:n] == 0).all())
+
+
+def test_no_alloc_mat_vec_refuses_a_second_stream_while_the_first_is_busy(q8):
+    # the built-in array serves one stream at a time, like the allocated scratch
+    lib = q8._lib.lib()
+    n, k = 4096, 14336
+    w = torch.zeros(q8.tiled_bytes(n, k), dtype=torch.uint8, device="cuda")
+    x = torch.ones(k, dtype=torch.float32, device="cuda")
+    y_a = torch.empty(n, dtype=torch.float32, device="cuda")
+    y_b = torch.full((n,), 7.0, dtype=torch.float32, device="cuda")
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    rc, still_running, batch = None, False, 300
+    while not still_running and batch <= 30000:
+        a.synchronize()
+        for _ in range(batch):
+            assert lib.nh_q8_0_gemv_tiled_f32_noalloc(w.data_ptr(), x.data_ptr(), y_a.data_ptr(), n, k, a.cuda_stream) == 0
+        rc = lib.nh_q8_0_gemv_tiled_f32_noalloc(w.data_ptr(), x.data_ptr(), y_b.data_ptr(), n, k, b.cuda_stream)
+        still_running = not a.query()
+        if rc == 0:
+            b.synchronize()
+            y_b.fill_(7.0)
+            torch.cuda.synchronize()
+        batch *= 10
+    if not still_running:
+        pytest.skip("stream a drains faster than this host enqueues: the overlap could not be set up")
+    assert rc == -10, rc  # NH_ERR_BUSY
+    torch.cuda.synchronize()
+    assert bool((y_b == 7.0).all())  # nothing was launched
+    assert lib.nh_q8_0_gemv_tiled_f32_noalloc(w.data_ptr(), x.data_ptr(), y_b.data_ptr(), n, k, b.cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert bool((y_b == 0).all())
+
+
 def test_no_alloc_mat_vec_matches_the_allocating_one(q8, oracle):
     lib = q8._lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
