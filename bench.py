@@ -273,6 +273,20 @@ def main() -> int:
         pre = side_workload("prefill", 100, 10)
         result["prefill"] = {"metric": pre["metric"], "value": pre["value"], "unit": pre["unit"], "ms_per_step": pre["ms_per_step"], "config": pre["config"], "roofline": pre["roofline"]}
         torch.cuda.empty_cache()
+        # the third named kernel (stand-alone activation quantize) and the two other benchmark configurations, compact
+        qz = side_workload("quantize", 100, 10)
+        result["quantize"] = {"config": qz["config"], "roofline": qz["roofline"], "fused_forms": qz["fused_forms"]}
+        cross = side_workload("crossover", 100, 10)
+        result["crossover"] = {"workload": cross["config"]["workload"], "unit": "us per nh_q8_0_mul_mat call (activation quantize included)",
+                               "rows": [{k: r[k] for k in ("M", "N", "K", "us", "kernel", "pct_hbm", "pct_mfma")} for r in cross["rows"]]}
+        torch.cuda.empty_cache()
+        l70 = side_workload("llama70b", 100, 10)
+        result["llama70b"] = {"workload": l70["config"]["workload"], "unit": "us per nh_q8_0_mul_mat call; pct_hbm = weight bytes / time against 8 TB/s",
+                              "rows": [{k: r[k] for k in ("projection", "M", "N", "K", "us", "kernel", "pct_hbm")} for r in l70["rows"]]}
+        torch.cuda.empty_cache()
+        probe = machine_probe("coissue_probe")
+        if probe is not None:
+            result["coissue"] = probe
     if not args.no_decode:
         result["decode"] = decode_step(args.decode_tokens)
         torch.cuda.empty_cache()
@@ -307,6 +321,25 @@ def dispatch_surface() -> dict | None:
         return None
     try:
         res = subprocess.run([exe, "30", "3"], capture_output=True, text=True, timeout=180)
+        line = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+        if res.returncode != 0 or not line:
+            return {"error": (res.stdout + res.stderr)[-400:], "returncode": res.returncode}
+        return json.loads(line[-1])
+    except (subprocess.TimeoutExpired, OSError, ValueError) as e:
+        return {"error": repr(e)[:400]}
+
+
+def machine_probe(name: str, *argv: str) -> dict | None:
+    """Runs one of the stand-alone HIP measurement programs built beside the host tests (tests/cpp/<name>.hip: read_probe, the
+    cost of a bare read of N bytes; coissue_probe, whether matrix pipe and VALU of a SIMD overlap) as a child process and returns
+    the JSON object it prints.  None when it has not been built."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "cpp", name)
+    if not os.path.exists(exe):
+        return None
+    try:
+        res = subprocess.run([exe, *argv], capture_output=True, text=True, timeout=120)
         line = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
         if res.returncode != 0 or not line:
             return {"error": (res.stdout + res.stderr)[-400:], "returncode": res.returncode}
@@ -387,6 +420,16 @@ def gemv_shapes(steps: int) -> dict:
         out[name] = row
         del sets, wps
         torch.cuda.empty_cache()
+    # the floor under each figure: a bare read of the same weight bytes (tests/cpp/read_probe.hip, a child process of its own)
+    torch.cuda.synchronize()
+    sizes = {name: sum(weight_bytes(n, k) for n in ns) for name, ns, k in shapes}
+    probe = machine_probe("read_probe", *[str(b) for b in sizes.values()])
+    if probe is not None and "reads" in probe:
+        for (name, _), rd in zip(sizes.items(), probe["reads"]):
+            out[name]["bare_read"] = {"us": rd["us"], "frac_of_hbm_peak": round(rd["GBs"] / HBM_PEAK_GBS, 4), "note": "one-shot read of the weight bytes alone, same workgroup size, HBM-cold"}
+            out[name]["cold"]["over_bare_read_us"] = round(out[name]["cold"]["avg_launch_us"] - rd["us"], 3)
+    elif probe is not None:
+        out["bare_read_error"] = probe
     return out
 
 
@@ -489,7 +532,7 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                 torch.cuda.synchronize()
                 sec = (time.perf_counter() - t0) / steps
                 wbytes = n * (k // 32) * 34
-                rows.append({"M": m, "N": n, "K": k, "us": round(sec * 1e6, 2), "weight_GBs": round(wbytes / sec / 1e9, 1), "TOPs": round(2.0 * m * n * k / sec / 1e12, 2),
+                rows.append({"M": m, "N": n, "K": k, "kernel": q8_0.plan_mul_mat(m, n, k)["kernel"], "us": round(sec * 1e6, 2), "weight_GBs": round(wbytes / sec / 1e9, 1), "TOPs": round(2.0 * m * n * k / sec / 1e12, 2),
                              "pct_hbm": round(100 * wbytes / sec / 1e9 / HBM_PEAK_GBS, 1), "pct_mfma": round(100 * 2.0 * m * n * k / sec / 1e12 / INT8_MFMA_PEAK_TOPS, 2)})
         return {"metric": "Q8_0 mul_mat (quantize + mat-vec / mat-mat) time against M", "unit": "us", "n_gpus": 1, "steps": steps, "warmup": warmup, "higher_is_better": False,
                 "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate", "data": "synthetic",
@@ -527,7 +570,7 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                     fn()
                 torch.cuda.synchronize()
                 sec = (time.perf_counter() - t0) / steps
-                rows.append({"projection": name, "M": m, "N": n, "K": k, "us": round(sec * 1e6, 2), "weight_GBs": round(wbytes / sec / 1e9, 1),
+                rows.append({"projection": name, "M": m, "N": n, "K": k, "kernel": q8_0.plan_mul_mat(m, n, k)["kernel"], "us": round(sec * 1e6, 2), "weight_GBs": round(wbytes / sec / 1e9, 1),
                              "pct_hbm": round(100 * wbytes / sec / 1e9 / HBM_PEAK_GBS, 1), "TOPs": round(2.0 * m * n * k / sec / 1e12, 2)})
             del ws
             torch.cuda.empty_cache()
@@ -602,13 +645,23 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
     ops = sum(2.0 * M * n * k for n, k in shapes)
     wall, ksec, n_l = timed(2, fn, len(shapes))
     ach = (ops / len(shapes)) / ksec / 1e12
+    # the shader clock the chip holds under this load: one wave on a stream of its own counts clocks for 2 ms beside a queue of
+    # the same launches (the published peak assumes 2.4 GHz)
+    for _ in range(60):
+        fn()
+    mhz = C.c_double()
+    rc_clk = lib.nh_profile_shader_clock(C.byref(mhz), 2000)
+    torch.cuda.synchronize()
+    clock_mhz = round(mhz.value, 1) if rc_clk == 0 else None
     return {
         "metric": "Q8_0 prefill mat-mat TOP/s (int8 MFMA)", "value": round(ops / wall / 1e12, 1), "unit": "TOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "dtype": "int8 x int8 -> int32 block sums (MFMA), fp32 scale-accumulate", "data": "synthetic",
         "config": {"workload": "prefill mat-mat, M=512 quantized activations x Q8_0 W [4096x4096] and [14336x4096] (two launches per step)",
                    "clock_settle_s": 0.2},
         "roofline": {"bound": "mfma", "kernel": "nh::gemm_tiled_kernel<TM, DUMP=false>", "achieved": round(ach, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": round(ach / INT8_MFMA_PEAK_TOPS, 4), "traffic": None, "ops_per_launch": ops / len(shapes), "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n_l},
+                     "frac": round(ach / INT8_MFMA_PEAK_TOPS, 4), "traffic": None, "ops_per_launch": ops / len(shapes), "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n_l,
+                     "shader_clock_mhz_under_load": clock_mhz, "peak_assumes_mhz": 2400.0,
+                     "frac_at_held_clock": round(ach / (INT8_MFMA_PEAK_TOPS * clock_mhz / 2400.0), 4) if clock_mhz else None},
     }
 
 

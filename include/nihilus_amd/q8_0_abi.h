@@ -280,6 +280,11 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
  * returns the summed, smallest and largest kernel durations in milliseconds.  Process-wide; not for concurrent use. */
 int nh_profile_begin(int kernel_kind, int64_t max_launches);
 int nh_profile_end(double* host_total_ms, int64_t* host_launches, double* host_min_ms, double* host_max_ms);
+/* The shader clock the GPU holds right now, in MHz: one wavefront on a stream of its own counts shader clocks against the
+ * constant 100 MHz timer for spin_us microseconds (1 .. 100000) beside whatever the caller has queued on other streams, and
+ * the call returns when it is done.  The int8-MFMA peak is quoted at 2.4 GHz; under a matrix-bound launch the chip holds
+ * less, and a figure against that peak cannot be read without the clock.  Allocates 16 bytes for the duration of the call. */
+int nh_profile_shader_clock(double* host_mhz, int64_t spin_us);
 
 /* Parity instrumentation ------------------------------------------------------------------------ */
 

@@ -61,6 +61,7 @@ SIGNATURES = {
     "nh_q8_0_mul_mat_residual": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
     "nh_q8_0_mul_mat_batch": (_int, [_vp, _i64, _vp, _i64, _vp]),
     "nh_profile_begin": (_int, [_int, _i64]),
+    "nh_profile_shader_clock": (_int, [C.POINTER(C.c_double), _i64]),
     "nh_profile_end": (_int, [C.POINTER(C.c_double), C.POINTER(_i64), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "nh_q8_0_debug_block_sums": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "nh_q8_0_fill_weight_blocks": (_int, [_vp, _u64, _i64, _i64, _vp]),

@@ -45,7 +45,58 @@ bool profile_next(int kind, hipEvent_t* start, hipEvent_t* stop) {
 
 } // namespace nh
 
+namespace nh {
+// clock64 counts shader clocks, wall_clock64 a constant 100 MHz: one wave reads both, spins for `ticks` of the latter, reads both again
+__global__ void shader_clock_kernel(long long* out, long long ticks) {
+	const long long w0 = wall_clock64();
+	const long long c0 = clock64();
+	long long w1	   = w0;
+	while (w1 - w0 < ticks) {
+		__builtin_amdgcn_s_sleep(4);
+		w1 = wall_clock64();
+	}
+	const long long c1 = clock64();
+	if (threadIdx.x == 0) {
+		out[0] = c1 - c0;
+		out[1] = w1 - w0;
+	}
+}
+} // namespace nh
+
 extern "C" {
+
+int nh_profile_shader_clock(double* host_mhz, int64_t spin_us) {
+	if (!host_mhz || spin_us < 1 || spin_us > 100000) {
+		return NH_ERR_ARGUMENT;
+	}
+	// a stream of its own (default priority, not synchronised with the NULL stream), so that the wave runs beside whatever
+	// the caller has queued elsewhere: the clock read is the one the chip holds under that load
+	hipStream_t s = nullptr;
+	hipError_t e  = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+	if (e != hipSuccess) {
+		return static_cast<int>(e);
+	}
+	long long* dev = nullptr;
+	long long host[2] = { 0, 0 };
+	e = hipMalloc(&dev, sizeof(host));
+	if (e == hipSuccess) {
+		nh::shader_clock_kernel<<<dim3(1), dim3(64), 0, s>>>(dev, spin_us * 100);
+		e = hipGetLastError();
+	}
+	if (e == hipSuccess) {
+		e = hipMemcpyAsync(host, dev, sizeof(host), hipMemcpyDeviceToHost, s);
+	}
+	if (e == hipSuccess) {
+		e = hipStreamSynchronize(s);
+	}
+	(void)hipFree(dev);
+	(void)hipStreamDestroy(s);
+	if (e != hipSuccess) {
+		return static_cast<int>(e);
+	}
+	*host_mhz = host[1] > 0 ? static_cast<double>(host[0]) / static_cast<double>(host[1]) * 100.0 : 0.0;
+	return NH_OK;
+}
 
 int nh_profile_begin(int kernel_kind, int64_t max_launches) {
 	if (kernel_kind < 0 || kernel_kind >= nh::KIND_COUNT || max_launches <= 0 || max_launches > (1 << 20)) {

@@ -16,6 +16,8 @@ HOST_TEST_BIN = os.path.join(HERE, "test_mul_mat_dispatch")
 MEGA_TEST_BIN = os.path.join(HERE, "test_mega_dispatch")  # the live dispatch point (core_types key), run on the GPU
 REFERENCE_MODE_BIN = os.path.join(HERE, "test_reference_mode_compiles")  # the headers against the reference's own primary template
 LAUNCH_FLOOR_BIN = os.path.join(HERE, "launch_floor_probe")  # cost of a dispatch that does nothing (a HIP program of its own, no library)
+READ_PROBE_BIN = os.path.join(HERE, "read_probe")  # what a bare read of a matrix's bytes costs (a HIP program of its own, no library)
+COISSUE_PROBE_BIN = os.path.join(HERE, "coissue_probe")  # whether the matrix pipe and the VALU of a SIMD overlap (a HIP program of its own, no library)
 TIME_MEGA_BIN = os.path.join(HERE, "time_mega_dispatch")  # decode token timed through the dispatch point (links the library only, not the checker)
 
 
@@ -38,19 +40,22 @@ def _build_one(src: str, out: str, with_checker: bool = True) -> str:
     return out
 
 
-def _build_launch_floor_probe() -> str:
+def _build_probe(src: str, out: str, extra: tuple[str, ...] = ()) -> str:
+    """A stand-alone HIP measurement program (no library): the library's own device flags."""
     from nihilus_amd.build import hipcc
 
-    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++20", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           os.path.join(HERE, "launch_floor_probe.hip"), "-o", LAUNCH_FLOOR_BIN]
+    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++20", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", *extra,
+           os.path.join(HERE, src), "-o", out]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
-        raise RuntimeError(f"launch floor probe build failed:\n{' '.join(cmd)}\n{res.stderr}")
-    return LAUNCH_FLOOR_BIN
+        raise RuntimeError(f"probe build failed:\n{' '.join(cmd)}\n{res.stderr}")
+    return out
 
 
 def build_host_tests() -> str:
-    _build_launch_floor_probe()
+    _build_probe("launch_floor_probe.hip", LAUNCH_FLOOR_BIN)
+    _build_probe("read_probe.hip", READ_PROBE_BIN)
+    _build_probe("coissue_probe.hip", COISSUE_PROBE_BIN, ("-mllvm", "-amdgpu-mfma-vgpr-form"))
     _build_one("test_mega_dispatch.cpp", MEGA_TEST_BIN)
     _build_one("time_mega_dispatch.cpp", TIME_MEGA_BIN, with_checker=False)
     _build_one("test_reference_mode_compiles.cpp", REFERENCE_MODE_BIN)

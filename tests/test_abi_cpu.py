@@ -208,6 +208,33 @@ def test_launch_floor_probe_runs():
 
 
 @pytest.mark.gpu
+def test_read_probe_and_coissue_probe_run():
+    import json
+
+    b = _host_tests()
+    res = subprocess.run([b.READ_PROBE_BIN, "17825792", "62390272"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout + res.stderr
+    reads = json.loads(res.stdout.strip().splitlines()[-1])["reads"]
+    assert [r["bytes"] for r in reads] == [17825792, 62390272] and all(1000 < r["GBs"] < 8000 for r in reads)
+    res = subprocess.run([b.COISSUE_PROBE_BIN], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout + res.stderr
+    out = json.loads(res.stdout.strip().splitlines()[-1])
+    assert 28 < out["clocks_per_mfma"] < 40 and 1.5 < out["clocks_per_valu_instruction"] < 6
+    assert 0.5 < out["at_four_waves"]["fraction_of_sum"] <= 1.1
+
+
+@pytest.mark.gpu
+def test_shader_clock_can_be_read():
+    from nihilus_amd import _lib
+
+    lib = _lib.lib()
+    mhz = C.c_double()
+    assert lib.nh_profile_shader_clock(C.byref(mhz), 200) == 0
+    assert 300.0 < mhz.value < 3000.0, mhz.value
+    assert lib.nh_profile_shader_clock(None, 200) == -6 and lib.nh_profile_shader_clock(C.byref(mhz), 0) == -6
+
+
+@pytest.mark.gpu
 def test_decode_token_timed_through_the_dispatch_point():
     # the measurement's own entry through the C++ dispatch header: a whole LLaMA-3-8B-shaped token and the FFN core alone
     import json
