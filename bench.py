@@ -766,23 +766,61 @@ def decode_step(tokens: int) -> dict:
     eps = C.c_float(1e-5)
 
     def real_token():
+        rc = 0
         for wqkv, yqkv, nqkv, wo_p, wg_p, wu_p, wd_p in per_layer:
-            rc = lib.nh_q8_0_gemv_tiled_multi_norm_f32(wqkv, yqkv, nqkv, 3, hp, nwp, eps, H, stream)
+            rc = rc or lib.nh_q8_0_gemv_tiled_multi_norm_f32(wqkv, yqkv, nqkv, 3, hp, nwp, eps, H, stream)
             rc = rc or lib.nh_q8_0_gemv_tiled_residual_f32(wo_p, qp, h0p, hp, H, H, stream)
             rc = rc or lib.nh_q8_0_ffn_f32(wg_p, wu_p, wd_p, hp, nwp, eps, h0p, hp, F, H, H, stream)
-            if rc != 0:
-                _lib.check("real-flow decode layer", rc)
+        if rc != 0:
+            _lib.check("real-flow decode layer", rc)
         _lib.check("nh_q8_0_gemv_tiled_multi_norm_f32", lib.nh_q8_0_gemv_tiled_multi_norm_f32(one_w, one_y, one_n, 1, hp, nwp, eps, H, stream))
 
-    for _ in range(5):
-        real_token()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(tokens):
-        real_token()
-    torch.cuda.synchronize()
-    sec_r = (time.perf_counter() - t0) / tokens
+    def timed_tokens(fn) -> float:
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(tokens):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / tokens
+
+    sec_r = timed_tokens(real_token)
     real_ok = bool(torch.isfinite(logits).all())
+
+    # The same data flow with one launch per block (nh_q8_0_decode_layer_f32): [attn_out + residual -> norm -> gate/up -> SiLU*up ->
+    # down + residual -> norm -> the NEXT block's q/k/v], the attention being the only seam; the first block's q/k/v go ahead as a
+    # launch of their own and the last block's launch ends in norm -> lm_head: 33 launches per token.
+    ffn_inp = torch.empty(H, dtype=torch.float32, device=dev)
+    l_outs = [torch.empty(H, dtype=torch.float32, device=dev) for _ in range(2)]
+    chain_calls = []
+    x_ptr_c = h0p
+    for li in range(LAYERS):
+        wq, wk, wv, wo, wg, wu, wd = (weights[li * 7 + j] for j in range(7))
+        out = l_outs[li & 1]
+        if li + 1 < LAYERS:
+            nxt = per_layer[li + 1]
+            tail = (nxt[0], nxt[1], nxt[2], 3)
+        else:
+            tail = (one_w, one_y, one_n, 1)
+        chain_calls.append((wo.data_ptr(), qp, x_ptr_c, ffn_inp.data_ptr(), wg.data_ptr(), wu.data_ptr(), wd.data_ptr(), nwp, out.data_ptr(), tail[0], tail[1], tail[2], tail[3], nwp, eps, H, F, stream))
+        x_ptr_c = out.data_ptr()
+    first_qkv = per_layer[0]
+
+    def chained_token():
+        rc = lib.nh_q8_0_gemv_tiled_multi_norm_f32(first_qkv[0], first_qkv[1], first_qkv[2], 3, h0p, nwp, eps, H, stream)
+        for call in chain_calls:
+            rc = rc or lib.nh_q8_0_decode_layer_f32(*call)
+        if rc != 0:
+            _lib.check("chained decode token", rc)
+
+    sec_c = timed_tokens(chained_token)
+    chained_ok = bool(torch.isfinite(logits).all())
+    _lib.check("nh_profile_begin", lib.nh_profile_begin(1, 512))
+    chained_token()
+    tot_c, cnt_c, mn_c, mx_c = C.c_double(), C.c_int64(), C.c_double(), C.c_double()
+    _lib.check("nh_profile_end", lib.nh_profile_end(C.byref(tot_c), C.byref(cnt_c), C.byref(mn_c), C.byref(mx_c)))
+    layer_bytes = sum(n * (k // 32) * 34 for _, n, k in shapes)
     return {
         "tok_s": round(1.0 / sec, 1),
         "ms_per_token": round(sec * 1e3, 4),
@@ -796,6 +834,13 @@ def decode_step(tokens: int) -> dict:
         "independent": {"tok_s": round(1.0 / sec_i, 1), "ms_per_token": round(sec_i * 1e3, 4), "pct_of_hbm_peak": round(100.0 * wbytes / sec_i / 1e9 / HBM_PEAK_GBS, 2),
                         "launches_per_token": launches_i,
                         "note": "same list without the ordered marks: a layer's seven projections read resident vectors here, so they go out as one grouped launch"},
+        "chained": {"tok_s": round(1.0 / sec_c, 1), "ms_per_token": round(sec_c * 1e3, 4), "pct_of_hbm_peak": round(100.0 * wbytes / sec_c / 1e9 / HBM_PEAK_GBS, 2),
+                    "launches_per_token": int(cnt_c.value), "outputs_finite": chained_ok, "entry": "nh_q8_0_decode_layer_f32",
+                    "block_launch_us": round((tot_c.value - mn_c.value - mx_c.value) / max(1, cnt_c.value - 2) * 1e3, 3),
+                    "block_launch_frac_of_hbm_peak": round(layer_bytes / ((tot_c.value - mn_c.value - mx_c.value) / max(1, cnt_c.value - 2) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                    "note": "a model's data flow with ONE launch per block: [attn_out + residual -> norm -> gate/up -> SiLU*up -> down + residual -> norm -> the next block's "
+                            "q/k/v], the attention (stood in for by q) being the only seam; first q/k/v ahead as a launch of their own, the last block's launch ends in norm -> lm_head. "
+                            "block_launch_us: mean kernel time of the 31 mid-token launches (231.7 MB of weights each)"},
         "real_flow": {"tok_s": round(1.0 / sec_r, 1), "ms_per_token": round(sec_r * 1e3, 4), "pct_of_hbm_peak": round(100.0 * wbytes / sec_r / 1e9 / HBM_PEAK_GBS, 2),
                       "launches_per_token": LAYERS * 3 + 1, "outputs_finite": real_ok,
                       "note": "the same weights with a model's data flow: per layer [norm -> q/k/v], [o + residual], [norm -> gate/up -> SiLU*up -> down + residual] as three "

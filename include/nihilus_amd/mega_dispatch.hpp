@@ -18,8 +18,14 @@
 //                                                                                                      infra/core_traits.hpp:971-995
 //   core_types::final_norm_and_sampling           rms_norm -> mul(output_norm) -> logits mul_mat      infra/core_traits.hpp:1186-1193
 //
-// eval_time bodies are one launch each (the quantize, the norm, SiLU * up and the residual add live inside the mat-vec
-// kernels); prompt_eval_time bodies quantize into a workspace and run the int8-MFMA mat-mat.
+// eval_time: the mat-vecs from one attention to the next are ONE launch (nh_q8_0_decode_layer_f32): mega_attention_apply runs the
+// attention hook and leaves its attn_out projection to mega_ffn, whose launch is [attn_out + residual -> norm -> gate/up -> SiLU * up ->
+// down + residual -> norm -> the NEXT block's q / k / v] (behind the last block: -> the logits); mega_qkv_prep_and_cache_publish of the
+// next block and final_norm_and_sampling then find their mat-vecs done and run only their hooks.  Per token: the first block's q / k / v
+// plus one launch per block, where the reference's fold makes three synchronous launches per block (cuda/thread_pool.hpp:46-67).  A
+// config that needs every core's outputs complete when that core returns declares `static constexpr bool amd_decode_per_core_launches
+// = true` and gets one launch per core instead (the quantize, the norm, SiLU * up and the residual add inside the mat-vec kernels).
+// prompt_eval_time bodies quantize into a workspace and run the int8-MFMA mat-mat.
 //
 // What those cores hold besides mat-muls is outside this path and is reached through three customisation points that a
 // config MUST specialise: without them a model runs and produces garbage (no rope, no cache write, q standing in for the
@@ -118,6 +124,31 @@ namespace nihilus {
 				return false;
 			}
 		}();
+
+		// eval_time chains a block's mat-vecs into one launch unless the config asks for one launch per core.
+		template<typename config_type> inline constexpr bool chains_decode = [] {
+			if constexpr (requires { config_type::amd_decode_per_core_launches; }) {
+				return !static_cast<bool>(config_type::amd_decode_per_core_launches);
+			} else {
+				return true;
+			}
+		}();
+		// What the eval_time cores hand to each other when they chain (one host thread drives the GPU, cuda/thread_pool.hpp:46-67):
+		// the attn_out projection that mega_attention_apply left to mega_ffn, and which mat-vecs a launch has already done for the
+		// core that comes next.
+		template<typename config_type> struct decode_chain_state {
+			int64_t attn_block{ -1 }; // block whose attn_out projection is pending; its operands:
+			const void* w_o{};
+			const float* attn{};
+			const float* layer_in{};
+			float* ffn_inp{};
+			int64_t qkv_done_block{ -1 }; // block whose q / k / v the previous block's launch has computed
+			bool logits_done{}; // the last block's launch has computed the logits
+			static decode_chain_state& get() {
+				static decode_chain_state state{};
+				return state;
+			}
+		};
 
 		// The input of transformer block `current_block`: token embeddings for the first, the previous block's l_out afterwards.
 		template<typename core_traits_type> inline const float* layer_input(core_traits_type& params, int64_t current_block) {
@@ -240,9 +271,16 @@ namespace nihilus {
 			float* outputs[3]	  = { q, k, v };
 			const int64_t ns[3]	  = { n_embd, n_kv, n_kv };
 			if constexpr (processing_phase == processing_phases::eval_time) {
-				amd_detail::check<config_type>(nh_q8_0_gemv_tiled_multi_norm_f32(weights, outputs, ns, 3, x, norm_w, mtt::layer_norm_rms_epsilon, n_embd, nullptr),
-					"mega_qkv eval_time: norm + q/k/v mat-vec");
+				auto& chain = amd_detail::decode_chain_state<config_type>::get();
+				if (amd_detail::chains_decode<config_type> && chain.qkv_done_block == current_block) {
+					// the previous block's launch ended in this block's norm + q / k / v (same operands, same outputs): only the hook is left
+				} else {
+					amd_detail::check<config_type>(nh_q8_0_gemv_tiled_multi_norm_f32(weights, outputs, ns, 3, x, norm_w, mtt::layer_norm_rms_epsilon, n_embd, nullptr),
+						"mega_qkv eval_time: norm + q/k/v mat-vec");
+				}
+				chain.qkv_done_block = -1;
 			} else {
+				amd_detail::decode_chain_state<config_type>::get() = {}; // a prompt pass ends whatever a decode step had pending
 				void* xq = amd_detail::workspace<config_type>(amd_detail::slot_quantized, nh_q8_0_tiled_bytes(rows, n_embd));
 				amd_detail::check<config_type>(nh_q8_0_rms_norm_quantize_tiled(x, norm_w, mtt::layer_norm_rms_epsilon, xq, rows, n_embd, nullptr), "mega_qkv prompt_eval_time: norm + quantize");
 				for (int i = 0; i < 3; ++i) {
@@ -286,7 +324,15 @@ namespace nihilus {
 			const float* residual = ptrs.template get_inp_embd_data<float>();
 			float* y			 = ptrs.template get_ffn_inp_data<float>();
 			const void* w		 = ptrs.template get_attn_output_w_data<void>();
-			if constexpr (processing_phase == processing_phases::eval_time) {
+			if constexpr (processing_phase == processing_phases::eval_time && amd_detail::chains_decode<config_type>) {
+				// left to mega_ffn of this block, whose launch starts with this projection
+				auto& chain	   = amd_detail::decode_chain_state<config_type>::get();
+				chain.attn_block = current_block;
+				chain.w_o		 = w;
+				chain.attn		 = attn;
+				chain.layer_in	 = residual;
+				chain.ffn_inp	 = y;
+			} else if constexpr (processing_phase == processing_phases::eval_time) {
 				amd_detail::check<config_type>(nh_q8_0_gemv_tiled_residual_f32(w, attn, residual, y, n_embd, n_embd, nullptr), "mega_attention_apply eval_time: attn_out mat-vec + residual");
 			} else {
 				const int64_t ws_bytes = nh_q8_0_mul_mat_workspace_bytes(rows, n_embd);
@@ -332,8 +378,49 @@ namespace nihilus {
 			const void* w_down	= ptrs.template get_ffn_down_w_data<void>();
 			float* y			= ptrs.template get_l_out_data<float>();
 			if constexpr (processing_phase == processing_phases::eval_time) {
-				// norm, gate / up, SiLU * up, quantize, down and the residual add (residual = the FFN's own input) as one launch
-				amd_detail::check<config_type>(nh_q8_0_ffn_f32(w_gate, w_up, w_down, x, norm_w, mtt::layer_norm_rms_epsilon, x, y, n_ff, n_embd, n_embd, nullptr), "mega_ffn eval_time");
+				auto& chain = amd_detail::decode_chain_state<config_type>::get();
+				if (amd_detail::chains_decode<config_type> && chain.attn_block == current_block && chain.ffn_inp == x) {
+					// attn_out + residual, this core, and what the next core starts with, as one launch
+					static constexpr int64_t n_kv	   = mtt::n_embd_kv_gqa;
+					static constexpr int64_t n_blocks  = mtt::block_count;
+					const void* next_w[3]			   = {};
+					float* next_y[3]				   = {};
+					int64_t next_n[3]				   = {};
+					int64_t next_count				   = 0;
+					const float* next_norm			   = nullptr;
+					if (current_block + 1 < n_blocks) {
+						auto& qkv_core = get_adjacent_value<cfg, core_types::mega_qkv_prep_and_cache_publish>::impl(params);
+						auto& q_out_op = qkv_core.values.template get_core<mega_qkv_prep_and_cache_publish_types, mega_qkv_prep_and_cache_publish_types::q_out>();
+						next_w[0]	   = amd_detail::data_of(weights_core.values.template get_core<weight_types, weight_types::attn_q>(), current_block + 1);
+						next_w[1]	   = amd_detail::data_of(weights_core.values.template get_core<weight_types, weight_types::attn_k>(), current_block + 1);
+						next_w[2]	   = amd_detail::data_of(weights_core.values.template get_core<weight_types, weight_types::attn_v>(), current_block + 1);
+						next_y[0]	   = q_out_op.template get_data<float>();
+						next_y[1]	   = static_cast<float*>(amd_detail::workspace<config_type>(amd_detail::slot_k, n_kv * 4));
+						next_y[2]	   = static_cast<float*>(amd_detail::workspace<config_type>(amd_detail::slot_v, n_kv * 4));
+						next_n[0]	   = n_embd;
+						next_n[1] = next_n[2] = n_kv;
+						next_count			  = 3;
+						next_norm = static_cast<const float*>(static_cast<const void*>(amd_detail::data_of(weights_core.values.template get_core<weight_types, weight_types::attn_norm>(), current_block + 1)));
+					} else {
+						next_w[0]  = weights_core.values.template get_core<weight_types, weight_types::output>().get_data();
+						next_y[0]  = static_cast<float*>(amd_detail::workspace<config_type>(amd_detail::slot_logits, static_cast<int64_t>(mtt::vocab_size) * 4));
+						next_n[0]  = mtt::vocab_size;
+						next_count = 1;
+						next_norm  = static_cast<const float*>(static_cast<const void*>(weights_core.values.template get_core<weight_types, weight_types::output_norm>().get_data()));
+					}
+					amd_detail::check<config_type>(nh_q8_0_decode_layer_f32(chain.w_o, chain.attn, chain.layer_in, chain.ffn_inp, w_gate, w_up, w_down, norm_w, y, next_w, next_y, next_n, next_count,
+													   next_norm, mtt::layer_norm_rms_epsilon, n_embd, n_ff, nullptr),
+						"mega_ffn eval_time: attn_out + ffn + next projections");
+					chain.attn_block = -1;
+					if (current_block + 1 < n_blocks) {
+						chain.qkv_done_block = current_block + 1;
+					} else {
+						chain.logits_done = true;
+					}
+				} else {
+					// norm, gate / up, SiLU * up, quantize, down and the residual add (residual = the FFN's own input) as one launch
+					amd_detail::check<config_type>(nh_q8_0_ffn_f32(w_gate, w_up, w_down, x, norm_w, mtt::layer_norm_rms_epsilon, x, y, n_ff, n_embd, n_embd, nullptr), "mega_ffn eval_time");
+				}
 			} else {
 				const int64_t rows = static_cast<int64_t>(sequence_length);
 				const int64_t q_bytes = nh_q8_0_tiled_bytes(rows, n_embd) > nh_q8_0_tiled_bytes(rows, n_ff) ? nh_q8_0_tiled_bytes(rows, n_embd) : nh_q8_0_tiled_bytes(rows, n_ff);
@@ -389,7 +476,13 @@ namespace nihilus {
 			const void* w		= ptrs.template get_output_w_data<void>();
 			float* logits		= static_cast<float*>(amd_detail::workspace<config_type>(amd_detail::slot_logits, vocab * 4));
 			const int64_t n		= vocab;
-			amd_detail::check<config_type>(nh_q8_0_gemv_tiled_multi_norm_f32(&w, &logits, &n, 1, x, norm_w, mtt::layer_norm_rms_epsilon, n_embd, nullptr), "final_norm_and_sampling: norm + logits mat-vec");
+			auto& chain = amd_detail::decode_chain_state<config_type>::get();
+			if (processing_phase == processing_phases::eval_time && amd_detail::chains_decode<config_type> && chain.logits_done) {
+				// the last block's launch ended in this norm + mat-vec (same operands, same output): only the hook is left
+			} else {
+				amd_detail::check<config_type>(nh_q8_0_gemv_tiled_multi_norm_f32(&w, &logits, &n, 1, x, norm_w, mtt::layer_norm_rms_epsilon, n_embd, nullptr), "final_norm_and_sampling: norm + logits mat-vec");
+			}
+			chain.logits_done = false;
 			amd_sampling<config_type>::impl(params, logits, nullptr);
 			// the host reads the sampled token next (infra/model.hpp, the generation loop): this core always waits
 			amd_detail::check<config_type>(nh_stream_sync(nullptr), "final_norm_and_sampling: stream sync");

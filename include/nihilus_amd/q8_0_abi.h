@@ -19,7 +19,7 @@
  *   Launches that hand data between workgroups do so through scratch memory that the library keeps per GPU (made on first
  *   use or by nh_q8_0_prepare): nh_q8_0_gemv_tiled*, nh_q8_0_gemv_tiled_group_f32, nh_q8_0_mul_mat*, nh_q8_0_mul_mat_batch,
  *   nh_q8_0_mul_mat_f32_activations (each when the shape makes them split K over workgroups), nh_q8_0_gemm_tiled* for M <= 64,
- *   and nh_q8_0_ffn_f32 always.  That scratch serves ONE stream at a time per GPU: enqueue such calls on one stream, or let
+ *   and nh_q8_0_ffn_f32 and nh_q8_0_decode_layer_f32 always.  That scratch serves ONE stream at a time per GPU: enqueue such calls on one stream, or let
  *   the other stream drain first.  A call that would use the scratch while a launch from a different stream may still be
  *   running returns NH_ERR_BUSY and launches nothing (not detected: work on a capturing stream, work that followed a
  *   launch on the NULL stream, and replays of captured graphs, which the caller must keep from overlapping).
@@ -204,6 +204,24 @@ int nh_q8_0_gemv_tiled_multi_norm_f32(const void* const* host_W_tiled, float* co
 #define NH_Q8_0_FFN_MAX_HIDDEN 65536
 int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled, const float* x, const float* norm_weight, float eps, const float* residual, float* y,
 	int64_t N_ff, int64_t K, int64_t N_out, void* stream);
+
+/* A transformer block's decode-time mat-vecs from one attention to the next as ONE launch:
+ *   ffn_inp = W_o . Q(attn) + layer_in                                      attn_out mul_mat -> residual add     (mega_attention_apply, infra/core_traits.hpp:768-772)
+ *   l_out   = W_down . Q(silu(W_gate . Q(n1)) * (W_up . Q(n1))) + ffn_inp   n1 = rms_norm(ffn_inp) * ffn_norm_weight   (mega_ffn, :971-995)
+ *   y_next[i] = W_next[i] . Q(n2),  i < count_next <= 3                     n2 = rms_norm(l_out) * next_norm_weight
+ * the last line being the NEXT block's q / k / v projections (mega_qkv_prep_and_cache_publish, :570-594) or, behind the last block,
+ * the logits (final_norm_and_sampling, :1186-1193); count_next == 0 leaves it out.  The reference runs these cores as separate
+ * synchronous launches per block (cuda/thread_pool.hpp:46-67); here the stages are ranges of one grid, and a stage's workgroups have
+ * their weight loads in flight while they wait for the stage before (see q8_0_decode_layer.hip).  Same arithmetic as
+ * nh_q8_0_gemv_tiled_residual_f32, nh_q8_0_ffn_f32 (norm and residual) and nh_q8_0_gemv_tiled_multi_norm_f32 run one after the other.
+ * W_o: [N_embd x N_embd] tiled; W_gate, W_up: [N_ff x N_embd]; W_down: [N_embd x N_ff]; W_next[i]: [N_next[i] x N_embd];
+ * attn, layer_in, ffn_inp, l_out: fp32 [N_embd]; y_next[i]: fp32 [N_next[i]]; host_* arrays are host memory, read before return.
+ * ffn_inp, l_out and every y_next must be distinct buffers (layer_in may be any of the inputs).  N_embd, N_ff multiples of 128.
+ * Shapes the one launch does not take (N_embd > 8192) and streams under HIP graph capture run the three launches instead.
+ * Uses the library's per-device scratch: two such calls must not overlap on one GPU (NH_ERR_BUSY, see "Streams"). */
+int nh_q8_0_decode_layer_f32(const void* W_o_tiled, const float* attn, const float* layer_in, float* ffn_inp, const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled,
+	const float* ffn_norm_weight, float* l_out, const void* const* host_W_next_tiled, float* const* host_y_next, const int64_t* host_N_next, int64_t count_next,
+	const float* next_norm_weight, float eps, int64_t N_embd, int64_t N_ff, void* stream);
 
 /* `count` INDEPENDENT mat-vecs, each with its own fp32 activation row, K and N (host arrays of device pointers and sizes;
  * host_residual or any entry of it may be NULL): y_i = W_i . quantize(x_i) [+ residual_i].  None of them may read or

@@ -329,6 +329,41 @@ int nh_q8_0_ffn_f32(const void* W_gate_tiled, const void* W_up_tiled, const void
 	return from_hip(nh::launch_ffn_decode(W_gate_tiled, W_up_tiled, W_down_tiled, x, norm_weight, eps, residual, y, N_ff, K, N_out, as_stream(stream)));
 }
 
+int nh_q8_0_decode_layer_f32(const void* W_o_tiled, const float* attn, const float* layer_in, float* ffn_inp, const void* W_gate_tiled, const void* W_up_tiled, const void* W_down_tiled,
+	const float* ffn_norm_weight, float* l_out, const void* const* host_W_next_tiled, float* const* host_y_next, const int64_t* host_N_next, int64_t count_next, const float* next_norm_weight,
+	float eps, int64_t N_embd, int64_t N_ff, void* stream) {
+	NH_TRY(check_shape(N_embd, 0, N_embd, true)); // attn_out: [N_embd x N_embd]; gate, up: [N_ff x N_embd]
+	NH_TRY(check_shape(N_embd, 0, N_ff, true)); // down: [N_embd x N_ff]
+	NH_REQUIRE(N_embd > 0 && N_ff > 0, NH_ERR_SHAPE);
+	NH_REQUIRE(N_ff <= NH_Q8_0_FFN_MAX_HIDDEN, NH_ERR_TOO_LARGE);
+	NH_REQUIRE(count_next >= 0 && count_next <= nh::GEMV_MAX_SEGMENTS, NH_ERR_ARGUMENT);
+	NH_REQUIRE(W_o_tiled && attn && layer_in && ffn_inp && W_gate_tiled && W_up_tiled && W_down_tiled && ffn_norm_weight && l_out, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(W_o_tiled) && aligned16(attn) && aligned16(layer_in) && aligned16(ffn_inp) && aligned16(W_gate_tiled) && aligned16(W_up_tiled) && aligned16(W_down_tiled) &&
+				   aligned16(ffn_norm_weight) && aligned16(l_out),
+		NH_ERR_ALIGNMENT);
+	NH_REQUIRE(eps >= 0.0f && eps < 1.0f, NH_ERR_ARGUMENT);
+	// ffn_inp and l_out are written by workgroups of different stages: as one buffer, which store lands last would be undefined
+	NH_REQUIRE(ffn_inp != l_out && attn != ffn_inp && attn != l_out, NH_ERR_ARGUMENT);
+	int64_t rows = 0;
+	if (count_next > 0) {
+		NH_REQUIRE(host_W_next_tiled && host_y_next && host_N_next && next_norm_weight, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(next_norm_weight), NH_ERR_ALIGNMENT);
+		for (int64_t i = 0; i < count_next; ++i) {
+			NH_REQUIRE(host_N_next[i] >= 0, NH_ERR_SHAPE);
+			if (host_N_next[i] > 0) {
+				NH_REQUIRE(host_W_next_tiled[i] && host_y_next[i], NH_ERR_NULL_POINTER);
+				NH_REQUIRE(aligned16(host_W_next_tiled[i]) && aligned16(host_y_next[i]), NH_ERR_ALIGNMENT);
+				NH_REQUIRE(host_y_next[i] != ffn_inp && host_y_next[i] != l_out, NH_ERR_ARGUMENT);
+			}
+			rows += host_N_next[i];
+		}
+		NH_REQUIRE(rows <= MAX_ROWS, NH_ERR_TOO_LARGE);
+	}
+	NH_TRY(require_device());
+	return from_hip(nh::launch_decode_layer(W_o_tiled, attn, layer_in, ffn_inp, W_gate_tiled, W_up_tiled, W_down_tiled, ffn_norm_weight, l_out, host_W_next_tiled, host_y_next, host_N_next,
+		rows > 0 ? static_cast<int>(count_next) : 0, next_norm_weight, eps, N_embd, N_ff, as_stream(stream)));
+}
+
 int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void* stream) {
 	NH_REQUIRE(N_ff >= 0, NH_ERR_SHAPE);
 	NH_REQUIRE(N_ff <= NH_Q8_0_FFN_MAX_HIDDEN, NH_ERR_TOO_LARGE);

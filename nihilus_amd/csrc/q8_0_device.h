@@ -269,6 +269,11 @@ hipError_t launch_gemv_tiled_f32_noalloc(const void* W, const float* x, float* y
 hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w_down, const float* x, const float* norm_w, float norm_eps, const float* residual, float* y, int64_t n_ff,
 	int64_t K, int64_t n_out, hipStream_t s);
 hipError_t copy_ffn_gate_up(float* gate_out, float* up_out, int64_t n_ff, hipStream_t s);
+// attn_out + residual -> norm -> gate/up -> SiLU * up -> down + residual -> norm -> up to GEMV_MAX_SEGMENTS projections, one launch where
+// the shape allows it (decode_layer_chains), else the three launches it stands for (q8_0_decode_layer.hip).  ffn_inp != l_out.
+bool decode_layer_chains(int64_t n_embd, int64_t n_ff, int64_t next_strips);
+hipError_t launch_decode_layer(const void* w_o, const float* attn, const float* layer_in, float* ffn_inp, const void* w_gate, const void* w_up, const void* w_down, const float* ffn_norm_w,
+	float* l_out, const void* const* w_next, float* const* y_next, const int64_t* n_next, int count_next, const float* next_norm_w, float eps, int64_t n_embd, int64_t n_ff, hipStream_t s);
 // Runs only the activation staging of the fused kernel and writes what it staged as packed blocks (parity check).
 hipError_t launch_gemv_dump_staged_x(const float* x, void* xq_blocks_out, int64_t K, hipStream_t s, const float* norm_w = nullptr, float norm_eps = 0.0f);
 // fp32 activations [M][K] against tiled Q8_0 weights without quantizing the activations (the reference's <float, block_q8_0, float>

@@ -257,7 +257,9 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch, hipStream_t s) {
 		void* p			   = nullptr;
 		const size_t blocks_end = static_cast<size_t>(GEMV_MAX_SPLIT_UNITS) * STRIP_ROWS * 8 + 2 * FFN_MAX_HIDDEN * 4 + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS * 8 + (FFN_MAX_HIDDEN / QK) * BLOCK_BYTES;
 		const size_t x_words_at = (blocks_end + 255) / 256 * 256;
-		const size_t bytes		= x_words_at + static_cast<size_t>(GEMV_SHARED_X_MAX_K / QK) * PUBLISHED_WORDS * 8;
+		const size_t rows_at	= x_words_at + static_cast<size_t>(GEMV_SHARED_X_MAX_K / QK) * PUBLISHED_WORDS * 8; // a multiple of 256
+		const size_t next_at	= rows_at + 2 * static_cast<size_t>(CHAIN_MAX_EMBD) * 8;
+		const size_t bytes		= next_at + static_cast<size_t>(CHAIN_MAX_EMBD / QK) * PUBLISHED_WORDS * 8;
 		e				   = hipMalloc(&p, bytes);
 		if (e != hipSuccess) {
 			return e;
@@ -277,6 +279,9 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch, hipStream_t s) {
 		sc.act_words  = reinterpret_cast<uint64_t*>(sc.gate_up + 2 * FFN_MAX_HIDDEN);
 		sc.act_blocks = reinterpret_cast<uint8_t*>(sc.act_words + (FFN_MAX_HIDDEN / STRIP_ROWS) * PUBLISHED_WORDS); // 16-byte aligned: every part before it is a multiple of 16 bytes
 		sc.x_words	  = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(p) + x_words_at);
+		sc.row_tagged[0] = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(p) + rows_at);
+		sc.row_tagged[1] = sc.row_tagged[0] + CHAIN_MAX_EMBD;
+		sc.x_words_next	 = reinterpret_cast<uint64_t*>(static_cast<uint8_t*>(p) + next_at);
 		sc.error_word = static_cast<unsigned*>(word);
 	}
 	if (next_epoch) {

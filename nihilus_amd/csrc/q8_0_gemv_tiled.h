@@ -445,6 +445,7 @@ __device__ __forceinline__ void split_k_finish(uint64_t* __restrict__ tagged, un
 constexpr int GEMV_MAX_SPLIT_UNITS	= 8192; // strips * splits when splits > 1
 constexpr int GEMV_MAX_SPLIT_STRIPS = 512;
 constexpr int FFN_MAX_HIDDEN		= 65536; // rows of the gate / up projections in a fused FFN launch
+constexpr int CHAIN_MAX_EMBD			= 8192; // longest hidden state the chained decode layer takes (a wave of its norm workgroups holds its share of the row in registers)
 constexpr int GEMV_SHARED_X_MAX_K	= 65536; // longest input row that a launch with a norm shares between its workgroups (longer: each works it out)
 // Sharing makes every other workgroup wait for the first strip's: a chain of row read, norm, quantize, publish and read-back
 // of ~3 us that the first round of workgroups sits out.  It pays once a launch runs several rounds, each of which would
@@ -459,6 +460,10 @@ struct gemv_scratch {
 	uint64_t* act_words = nullptr; // [FFN_MAX_HIDDEN / 32][PUBLISHED_WORDS] {epoch, payload}: the quantized activation of the down projection
 	uint8_t* act_blocks = nullptr; // [FFN_MAX_HIDDEN / 32] packed 34-byte blocks: the activation of the three-launch form used under graph capture
 	uint64_t* x_words	= nullptr; // [GEMV_SHARED_X_MAX_K / 32][PUBLISHED_WORDS] {epoch, payload}: a launch's normalised, quantized input row, from its first strip's workgroups to the rest
+	// the chained decode layer (q8_0_decode_layer.hip): the fp32 rows that one stage hands to the next as {epoch, value} words, and
+	// the second normalised, quantized row of the launch
+	uint64_t* row_tagged[2] = { nullptr, nullptr }; // [CHAIN_MAX_EMBD] each: attn_out + residual, then down + residual
+	uint64_t* x_words_next	= nullptr; // [CHAIN_MAX_EMBD / 32][PUBLISHED_WORDS]
 	unsigned epoch	   = 0; // with next_epoch = true: a value no earlier launch on this device has used
 	unsigned* error_word = nullptr; // 4 bytes of pinned host memory the device can write: non-zero once a kernel has given up a bounded wait
 	int spin_limit	   = PUBLISHED_SPIN_LIMIT; // polls before a consumer of published blocks gives up (lowered only by tests)

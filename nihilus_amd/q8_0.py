@@ -141,6 +141,25 @@ def ffn(w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, x: torch
     return y
 
 
+def decode_layer(w_o: torch.Tensor, attn: torch.Tensor, layer_in: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ffn_norm: torch.Tensor,
+                 w_next: list[torch.Tensor], n_next: list[int], next_norm: torch.Tensor | None, eps: float, n_embd: int, n_ff: int):
+    """One block's decode mat-vecs from one attention to the next (nh_q8_0_decode_layer_f32): returns (ffn_inp, l_out, [y_next...])."""
+    import ctypes
+
+    attn, layer_in, ffn_norm = _dev(attn, torch.float32, "attn"), _dev(layer_in, torch.float32, "layer_in"), _dev(ffn_norm, torch.float32, "ffn_norm")
+    ffn_inp = torch.empty(n_embd, dtype=torch.float32, device=attn.device)
+    l_out = torch.empty(n_embd, dtype=torch.float32, device=attn.device)
+    ys = [torch.empty(n, dtype=torch.float32, device=attn.device) for n in n_next]
+    cnt = len(w_next)
+    wp = (ctypes.c_void_p * max(cnt, 1))(*[w.data_ptr() for w in w_next])
+    yp = (ctypes.c_void_p * max(cnt, 1))(*[y.data_ptr() for y in ys])
+    np_ = (ctypes.c_int64 * max(cnt, 1))(*n_next)
+    _lib.check("nh_q8_0_decode_layer_f32", _lib.lib().nh_q8_0_decode_layer_f32(
+        w_o.data_ptr(), attn.data_ptr(), layer_in.data_ptr(), ffn_inp.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), ffn_norm.data_ptr(), l_out.data_ptr(),
+        wp, yp, np_, cnt, next_norm.data_ptr() if next_norm is not None else None, ctypes.c_float(eps), n_embd, n_ff, _stream()))
+    return ffn_inp, l_out, ys
+
+
 def debug_ffn_gate_up(n_ff: int):
     """The gate and up outputs (fp32 [n_ff] each) of the last ffn() on this device."""
     g = torch.empty(n_ff, dtype=torch.float32, device="cuda")

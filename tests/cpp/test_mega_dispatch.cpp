@@ -10,6 +10,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 extern "C" { // the CPU checker
@@ -121,11 +122,24 @@ static std::vector<float> cpu_mul_mat(const matrix& w, const std::vector<float>&
 	return c;
 }
 
-template<processing_phases phase> static int run_phase(nihilus_cathedral<mock_config>& model, const matrix (&wq)[2], const matrix (&wk)[2], const matrix (&wv)[2], const matrix (&wo)[2],
+// the mat-mul path alone, one launch per core in the decode phase too (every core's outputs complete when it returns)
+struct per_core_config : mock_config {
+	static constexpr bool amd_decode_per_core_launches{ true };
+};
+template<> struct nihilus::amd_qkv_epilogue<per_core_config> : nihilus::amd_qkv_epilogue<mock_config> {};
+template<> struct nihilus::amd_sampling<per_core_config> : nihilus::amd_sampling<mock_config> {};
+
+template<processing_phases phase, typename dispatch_config = mock_config> static int run_phase(nihilus_cathedral<mock_config>& model, const matrix (&wq)[2], const matrix (&wk)[2], const matrix (&wv)[2], const matrix (&wo)[2],
 	const matrix (&wg)[2], const matrix (&wu)[2], const matrix (&wd)[2], const matrix& w_out, const std::vector<float> (&attn_norm)[2], const std::vector<float> (&ffn_norm)[2],
 	const std::vector<float>& out_norm, const std::vector<float>& x0, int64_t rows, void* d_q, void* d_ffn_inp, void* d_l_out) {
 	constexpr int64_t E = mtt::embedding_length, KV = mtt::n_embd_kv_gqa, F = mtt::feed_forward_length, V = mtt::vocab_size;
-	const char* name = phase == processing_phases::eval_time ? "eval_time" : "prompt_eval_time";
+	// in the decode phase the cores chain (unless the config asks for one launch per core): mega_attention_apply leaves its projection
+	// to mega_ffn, whose launch also does the next core's mat-vecs, so ffn_inp is complete after mega_ffn, not before
+	constexpr bool chained = phase == processing_phases::eval_time && amd_detail::chains_decode<dispatch_config>;
+	const char* name = phase == processing_phases::eval_time ? (chained ? "eval_time (chained)" : "eval_time (per core)") : "prompt_eval_time";
+	auto dispatch = [&]<core_types core, typename core_type>(core_type& c, int64_t block) {
+		kernel_dispatcher_impl<dispatch_config, core_type, device_types::gpu, gfx950_arch_index, core, phase>::impl(c, block);
+	};
 	auto& qkv		 = static_cast<qkv_core&>(model);
 	auto& attn		 = static_cast<attn_core&>(model);
 	auto& ffn		 = static_cast<ffn_core&>(model);
@@ -137,7 +151,11 @@ template<processing_phases phase> static int run_phase(nihilus_cathedral<mock_co
 
 	std::vector<float> layer_in = x0, got, got_k, got_v;
 	for (int64_t block = 0; block < 2; ++block) {
-		kernel_dispatcher<mock_config, phase, qkv_core>::impl(qkv, block);
+		if constexpr (std::is_same_v<dispatch_config, mock_config>) {
+			kernel_dispatcher<mock_config, phase, qkv_core>::impl(qkv, block); // the reference's caller-side template picks the specialisation
+		} else {
+			dispatch.template operator()<core_types::mega_qkv_prep_and_cache_publish>(qkv, block);
+		}
 		REQUIRE(seen_rows == static_cast<uint64_t>(rows) && seen_k && seen_v);
 		REQUIRE(download(got, d_q, rows * E) == 0 && download(got_k, seen_k, rows * KV) == 0 && download(got_v, seen_v, rows * KV) == 0);
 		const double eq = rel_l2(got, cpu_mul_mat(wq[block], layer_in, rows, &attn_norm[block], nullptr));
@@ -147,14 +165,19 @@ template<processing_phases phase> static int run_phase(nihilus_cathedral<mock_co
 		REQUIRE(eq <= 1e-4 && ek <= 1e-4 && ev <= 1e-4);
 
 		const std::vector<float> q_gpu = got; // the stand-in attention output of the primary amd_attention
-		kernel_dispatcher<mock_config, phase, attn_core>::impl(attn, block);
-		REQUIRE(download(got, d_ffn_inp, rows * E) == 0);
+		dispatch.template operator()<core_types::mega_attention_apply>(attn, block);
+		if constexpr (!chained) {
+			REQUIRE(download(got, d_ffn_inp, rows * E) == 0);
+		}
+		dispatch.template operator()<core_types::mega_ffn>(ffn, block);
+		if constexpr (chained) {
+			REQUIRE(download(got, d_ffn_inp, rows * E) == 0);
+		}
 		const double eo = rel_l2(got, cpu_mul_mat(wo[block], q_gpu, rows, nullptr, &layer_in));
 		std::printf("%s block %lld mega_attention  attn_out + residual %.2e\n", name, static_cast<long long>(block), eo);
 		REQUIRE(eo <= 1e-4);
 
 		const std::vector<float> ffn_in = got;
-		kernel_dispatcher<mock_config, phase, ffn_core>::impl(ffn, block);
 		REQUIRE(download(got, d_l_out, rows * E) == 0);
 		const std::vector<float> g = cpu_mul_mat(wg[block], ffn_in, rows, &ffn_norm[block], nullptr), u = cpu_mul_mat(wu[block], ffn_in, rows, &ffn_norm[block], nullptr);
 		std::vector<uint8_t> hq(rows * (F / 32) * 34);
@@ -171,7 +194,8 @@ template<processing_phases phase> static int run_phase(nihilus_cathedral<mock_co
 		REQUIRE(ef <= 1e-3);
 		layer_in = got;
 	}
-	kernel_dispatcher<mock_config, phase, final_core>::impl(fin);
+	seen_logits = nullptr;
+	kernel_dispatcher_impl<dispatch_config, final_core, device_types::gpu, gfx950_arch_index, core_types::final_norm_and_sampling, phase>::impl(fin);
 	REQUIRE(seen_logits);
 	REQUIRE(download(got, seen_logits, V) == 0);
 	const std::vector<float> last(layer_in.end() - E, layer_in.end());
@@ -244,6 +268,11 @@ int main(int argc, char** argv) {
 	const std::vector<float> x_one(x0.begin(), x0.begin() + E);
 	REQUIRE(run_phase<processing_phases::eval_time>(model, wq, wk, wv, wo, wg, wu, wd, w_out, attn_norm, ffn_norm, out_norm, x_one, 1, d_q, d_ffn_inp, d_l_out) == 0);
 	REQUIRE(run_phase<processing_phases::prompt_eval_time>(model, wq, wk, wv, wo, wg, wu, wd, w_out, attn_norm, ffn_norm, out_norm, x0, ROWS, d_q, d_ffn_inp, d_l_out) == 0);
+	// a decode step right after a prompt pass (nothing of the prompt pass may be taken for a finished decode mat-vec), then the
+	// same step with one launch per core
+	REQUIRE(run_phase<processing_phases::eval_time>(model, wq, wk, wv, wo, wg, wu, wd, w_out, attn_norm, ffn_norm, out_norm, x_one, 1, d_q, d_ffn_inp, d_l_out) == 0);
+	amd_prepare<per_core_config, mtt>(1);
+	REQUIRE((run_phase<processing_phases::eval_time, per_core_config>(model, wq, wk, wv, wo, wg, wu, wd, w_out, attn_norm, ffn_norm, out_norm, x_one, 1, d_q, d_ffn_inp, d_l_out) == 0));
 
 	// a long prompt after a short one, and nothing was allocated on the way; preparing again for the same length allocates nothing either
 	REQUIRE(amd_workspace_allocations<mock_config>() == allocations_after_prepare);

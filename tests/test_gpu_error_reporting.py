@@ -52,6 +52,40 @@ def test_ffn_timeout_is_reported_by_the_next_sync(q8, oracle):
     assert "bounded wait" in q8._lib.status_string(NH_ERR_DEVICE_TIMEOUT)
 
 
+def test_decode_layer_timeout_is_reported_and_every_stage_still_drains(q8):
+    # the chained decode layer hands data between five stages; with the poll limit at 1 every stage gives up on the one before,
+    # the outputs hold NaN, the error is reported, and the launch runs to its end
+    lib = q8._lib.lib()
+    n_embd, n_ff, nxt = 1024, 3584, [1024, 256, 256]
+    ws = {name: q8.tile(q8.fill_weight_blocks(40 + i, n, k), n, k) for i, (name, n, k) in enumerate(
+        [("o", n_embd, n_embd), ("g", n_ff, n_embd), ("u", n_ff, n_embd), ("d", n_embd, n_ff), ("q", 1024, n_embd), ("k", 256, n_embd), ("v", 256, n_embd)])}
+    attn, x = q8.fill_activations(50, n_embd), q8.fill_activations(51, n_embd)
+    norm = torch.ones(n_embd, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run():
+        return q8.decode_layer(ws["o"], attn, x, ws["g"], ws["u"], ws["d"], norm, [ws["q"], ws["k"], ws["v"]], nxt, norm, 1e-5, n_embd, n_ff)
+
+    h, y, outs = run()
+    assert lib.nh_stream_sync(stream) == 0 and all(bool(torch.isfinite(t).all()) for t in [h, y, *outs])
+    good = [to_host(t) for t in [h, y, *outs]]
+    os.environ["NH_Q8_0_DEBUG_HOOKS"] = "1"
+    try:
+        assert lib.nh_q8_0_debug_set_spin_limit(1) == 0
+        h2, y2, outs2 = run()
+        assert lib.nh_stream_sync(stream) == NH_ERR_DEVICE_TIMEOUT
+        assert bool(torch.isnan(y2).any()) or bool(torch.isnan(outs2[0]).any())
+        assert bool(torch.isfinite(h2).all())  # the first stage waits for nobody
+        assert lib.nh_q8_0_clear_error() == NH_ERR_DEVICE_TIMEOUT
+    finally:
+        assert lib.nh_q8_0_debug_set_spin_limit(1 << 20) == 0
+        os.environ.pop("NH_Q8_0_DEBUG_HOOKS", None)
+    h3, y3, outs3 = run()
+    assert lib.nh_stream_sync(stream) == 0
+    for a, b in zip(good, [to_host(t) for t in [h3, y3, *outs3]]):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_scratch_in_use_on_another_stream_is_refused(q8, oracle):
     lib = q8._lib.lib()
     n, k = 4096, 14336  # K split over four workgroups per strip: the hand-off goes through the per-GPU scratch
