@@ -65,7 +65,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU leg (for profiler runs)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the bounded CPU sample")
     ap.add_argument("--calibration-copies", type=int, default=0, help="run this many plain 64 MiB device copies first (a known-size kernel to scale hardware byte counters by)")
-    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "quantize", "get_rows", "crossover", "llama70b", "f32act"], default="ffn_decode",
+    ap.add_argument("--workload", choices=["ffn_decode", "prefill", "prefill_ffn", "quantize", "get_rows", "crossover", "llama70b", "f32act"], default="ffn_decode",
                     help="ffn_decode (default): the headline line.  prefill / quantize: side lines for the other two kernels "
                     "(M=512 int8-MFMA mat-mat against the MFMA roofline; M=512 activation quantize against HBM)")
     ap.add_argument("--ffn-mode", choices=["group", "two", "fused"], default="fused",
@@ -272,6 +272,9 @@ def main() -> int:
         result["gemv_shapes"] = gemv_shapes(min(args.steps, 400))
         pre = side_workload("prefill", 100, 10)
         result["prefill"] = {"metric": pre["metric"], "value": pre["value"], "unit": pre["unit"], "ms_per_step": pre["ms_per_step"], "config": pre["config"], "roofline": pre["roofline"]}
+        torch.cuda.empty_cache()
+        pf = side_workload("prefill_ffn", 100, 10)
+        result["prefill_ffn"] = {k: pf[k] for k in ("config", "three_launches_us", "five_launches_us", "speedup", "outputs_bit_identical", "TOPs", "pct_mfma")}
         torch.cuda.empty_cache()
         # the third named kernel (stand-alone activation quantize) and the two other benchmark configurations, compact
         qz = side_workload("quantize", 100, 10)
@@ -508,6 +511,56 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
             "roofline": {"bound": "hbm", "kernel": "nh::quantize_kernel<true>", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n},
         }
+
+    if kind == "prefill_ffn":
+        # the prompt-phase FFN of one block at M = 512, LLaMA-3-8B shapes, as the dispatch header's mega_ffn core issues it (three
+        # launches: norm + quantize; gate / up mat-mats with SiLU * up and the quantizer in their epilogue; down mat-mat + residual)
+        # against the five launches it replaced (two mat-mats writing fp32 [M x n_ff], a SiLU * up quantizer reading them back)
+        F = 14336
+        nw = q8_0.fill_activations(5, K)
+        wg, wu, wd = (q8_0.tile(q8_0.fill_weight_blocks(40 + i, n, k), n, k) for i, (n, k) in enumerate(((F, K), (F, K), (K, F))))
+        xq = torch.empty(q8_0.tiled_bytes(M, K), dtype=torch.uint8, device=x.device)
+        hq = torch.empty(q8_0.tiled_bytes(M, F), dtype=torch.uint8, device=x.device)
+        gate = torch.empty((M, F), dtype=torch.float32, device=x.device)
+        up = torch.empty_like(gate)
+        y = torch.empty((M, K), dtype=torch.float32, device=x.device)
+        eps = C.c_float(1e-5)
+        need = lib.nh_q8_0_gate_up_silu_workspace_bytes(M, F, K)
+
+        def five():
+            rc = lib.nh_q8_0_rms_norm_quantize_tiled(x.data_ptr(), nw.data_ptr(), eps, xq.data_ptr(), M, K, stream)
+            rc = rc or lib.nh_q8_0_gemm_tiled(wg.data_ptr(), xq.data_ptr(), gate.data_ptr(), M, F, K, stream)
+            rc = rc or lib.nh_q8_0_gemm_tiled(wu.data_ptr(), xq.data_ptr(), up.data_ptr(), M, F, K, stream)
+            rc = rc or lib.nh_q8_0_silu_mul_quantize_tiled(gate.data_ptr(), up.data_ptr(), hq.data_ptr(), M, F, stream)
+            rc = rc or lib.nh_q8_0_gemm_tiled_residual(wd.data_ptr(), hq.data_ptr(), x.data_ptr(), y.data_ptr(), M, K, F, stream)
+            _lib.check("prefill FFN, five launches", rc)
+
+        def three():
+            rc = lib.nh_q8_0_rms_norm_quantize_tiled(x.data_ptr(), nw.data_ptr(), eps, xq.data_ptr(), M, K, stream)
+            rc = rc or lib.nh_q8_0_gemm_tiled_gate_up_silu(wg.data_ptr(), wu.data_ptr(), xq.data_ptr(), hq.data_ptr(), None, 0, M, F, K, stream)
+            rc = rc or lib.nh_q8_0_gemm_tiled_residual(wd.data_ptr(), hq.data_ptr(), x.data_ptr(), y.data_ptr(), M, K, F, stream)
+            _lib.check("prefill FFN, three launches", rc)
+
+        def wall(fn):
+            warm_up(fn, 0.2)
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / steps
+
+        t5 = wall(five)
+        y5 = y.clone()
+        t3 = wall(three)
+        same = bool(torch.equal(y5, y))
+        t5b, t3b = wall(five), wall(three)  # once more in the other order: the clock the chip holds depends on what ran before
+        t5, t3 = min(t5, t5b), min(t3, t3b)
+        ops = 2.0 * M * K * F * 3
+        return {"metric": "Q8_0 prefill FFN (norm, gate/up, SiLU*up, down, residual) time at M=512", "value": round(t3 * 1e6, 2), "unit": "us", "n_gpus": 1, "steps": steps, "warmup": warmup,
+                "ms_per_step": round(t3 * 1e3, 6), "higher_is_better": False, "dtype": "int8 x int8 -> int32 block sums (MFMA), fp32 scale-accumulate", "data": "synthetic",
+                "config": {"workload": f"one block's prompt-phase FFN, M={M}, hidden {K}, n_ff {F}: three launches (fused gate/up kernel taken: {need == 0})"},
+                "three_launches_us": round(t3 * 1e6, 2), "five_launches_us": round(t5 * 1e6, 2), "speedup": round(t5 / t3, 4), "outputs_bit_identical": same,
+                "TOPs": round(ops / t3 / 1e12, 1), "pct_mfma": round(100 * ops / t3 / 1e12 / INT8_MFMA_PEAK_TOPS, 2)}
 
     if kind == "crossover":
         # M in {1, 2, 4, 8, 32, 64, 128, 512} against the same two weights: where the mat-vec (HBM-bound; M = 2, 3 still on it) hands over to the

@@ -59,7 +59,7 @@ namespace nihilus {
 		// (infra/behavioral_axes.hpp:61-90, infra/model.hpp:241).  Here the same happens in amd_prepare (below): every slot is
 		// sized once for the longest sequence the config allows, and the dispatchers only check capacity.  One host thread
 		// drives the GPU (cuda/thread_pool.hpp:46-67).
-		enum workspace_slot : int { slot_quantized = 0, slot_k, slot_v, slot_gate, slot_up, slot_attention, slot_logits, slot_count };
+		enum workspace_slot : int { slot_quantized = 0, slot_k, slot_v, slot_activation, slot_gate_up, slot_attention, slot_logits, slot_count };
 		struct workspace_entry {
 			void* ptr{};
 			int64_t bytes{};
@@ -175,14 +175,19 @@ namespace nihilus {
 		const int64_t rows	 = max_sequence_length < 1 ? 1 : static_cast<int64_t>(max_sequence_length);
 		const int64_t n_embd = model_traits_type::embedding_length, n_ff = model_traits_type::feed_forward_length, n_kv = model_traits_type::n_embd_kv_gqa;
 		int64_t quantized	 = nh_q8_0_tiled_bytes(rows, n_embd);
-		for (const int64_t other : { nh_q8_0_tiled_bytes(rows, n_ff), nh_q8_0_mul_mat_workspace_bytes(rows, n_embd), nh_q8_0_mul_mat_workspace_bytes(rows, n_ff) }) {
-			quantized = other > quantized ? other : quantized;
-		}
-		amd_detail::reserve_slot<config_type>(amd_detail::slot_quantized, quantized);
+		const int64_t other	 = nh_q8_0_mul_mat_workspace_bytes(rows, n_embd);
+		quantized			 = other > quantized ? other : quantized;
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_quantized, quantized); // activations quantized along the embedding
 		amd_detail::reserve_slot<config_type>(amd_detail::slot_k, rows * n_kv * 4);
 		amd_detail::reserve_slot<config_type>(amd_detail::slot_v, rows * n_kv * 4);
-		amd_detail::reserve_slot<config_type>(amd_detail::slot_gate, rows * n_ff * 4);
-		amd_detail::reserve_slot<config_type>(amd_detail::slot_up, rows * n_ff * 4);
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_activation, nh_q8_0_tiled_bytes(rows, n_ff)); // the down projection's quantized activation
+		// fp32 gate / up outputs of prompts too short for the fused gate / up kernel (longer ones need none)
+		int64_t gate_up = 0;
+		for (int64_t r = 1; r <= rows; ++r) {
+			const int64_t need = nh_q8_0_gate_up_silu_workspace_bytes(r, n_ff, n_embd);
+			gate_up			   = need > gate_up ? need : gate_up;
+		}
+		amd_detail::reserve_slot<config_type>(amd_detail::slot_gate_up, gate_up);
 		amd_detail::reserve_slot<config_type>(amd_detail::slot_attention, rows * n_embd * 4);
 		amd_detail::reserve_slot<config_type>(amd_detail::slot_logits, static_cast<int64_t>(model_traits_type::vocab_size) * 4);
 		amd_detail::check<config_type>(nh_q8_0_prepare(), "amd_prepare: library scratch");
@@ -423,15 +428,16 @@ namespace nihilus {
 				}
 			} else {
 				const int64_t rows = static_cast<int64_t>(sequence_length);
-				const int64_t q_bytes = nh_q8_0_tiled_bytes(rows, n_embd) > nh_q8_0_tiled_bytes(rows, n_ff) ? nh_q8_0_tiled_bytes(rows, n_embd) : nh_q8_0_tiled_bytes(rows, n_ff);
-				void* xq			  = amd_detail::workspace<config_type>(amd_detail::slot_quantized, q_bytes);
-				float* gate			  = static_cast<float*>(amd_detail::workspace<config_type>(amd_detail::slot_gate, rows * n_ff * 4));
-				float* up			  = static_cast<float*>(amd_detail::workspace<config_type>(amd_detail::slot_up, rows * n_ff * 4));
+				// three launches: norm + quantize; gate and up mat-mats with SiLU * up and the quantizer behind them (one launch, no fp32
+				// intermediates, where the shape takes the fused kernel: then gate_up_bytes is 0); down mat-mat with the residual in its store
+				void* xq					= amd_detail::workspace<config_type>(amd_detail::slot_quantized, nh_q8_0_tiled_bytes(rows, n_embd));
+				void* hq					= amd_detail::workspace<config_type>(amd_detail::slot_activation, nh_q8_0_tiled_bytes(rows, n_ff));
+				const int64_t gate_up_bytes = nh_q8_0_gate_up_silu_workspace_bytes(rows, n_ff, n_embd);
+				void* gate_up				= amd_detail::workspace<config_type>(amd_detail::slot_gate_up, gate_up_bytes);
 				amd_detail::check<config_type>(nh_q8_0_rms_norm_quantize_tiled(x, norm_w, mtt::layer_norm_rms_epsilon, xq, rows, n_embd, nullptr), "mega_ffn prompt_eval_time: norm + quantize");
-				amd_detail::check<config_type>(nh_q8_0_gemm_tiled(w_gate, xq, gate, rows, n_ff, n_embd, nullptr), "mega_ffn prompt_eval_time: gate mat-mat");
-				amd_detail::check<config_type>(nh_q8_0_gemm_tiled(w_up, xq, up, rows, n_ff, n_embd, nullptr), "mega_ffn prompt_eval_time: up mat-mat");
-				amd_detail::check<config_type>(nh_q8_0_silu_mul_quantize_tiled(gate, up, xq, rows, n_ff, nullptr), "mega_ffn prompt_eval_time: SiLU * up + quantize");
-				amd_detail::check<config_type>(nh_q8_0_gemm_tiled_residual(w_down, xq, x, y, rows, n_embd, n_ff, nullptr), "mega_ffn prompt_eval_time: down mat-mat + residual");
+				amd_detail::check<config_type>(nh_q8_0_gemm_tiled_gate_up_silu(w_gate, w_up, xq, hq, gate_up, gate_up_bytes, rows, n_ff, n_embd, nullptr),
+					"mega_ffn prompt_eval_time: gate / up mat-mats + SiLU * up + quantize");
+				amd_detail::check<config_type>(nh_q8_0_gemm_tiled_residual(w_down, hq, x, y, rows, n_embd, n_ff, nullptr), "mega_ffn prompt_eval_time: down mat-mat + residual");
 			}
 			amd_detail::after_launch<config_type>();
 		}

@@ -247,6 +247,18 @@ int nh_q8_0_gemm_tiled(const void* W_tiled, const void* Aq_tiled, float* C, int6
  * sum.  residual: fp32 [M][N], may be C itself (in-place accumulate). */
 int nh_q8_0_gemm_tiled_residual(const void* W_tiled, const void* Aq_tiled, const float* residual, float* C, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The prefill FFN's first half as one call: act = quantize_row_q8_0(silu(W_gate . Aq) * (W_up . Aq)), written in the tiled layout as the
+ * activation operand of the down projection (rows padded with zero blocks to a multiple of 32).  Stands for the ffn_gate and ffn_up
+ * mul_mat -> ffn_silu -> ffn_gate_par (mul) chain of the reference's mega_ffn core in the prompt phase (infra/core_traits.hpp:976-989).
+ * Where each matrix alone would take the prefill MFMA kernel it is ONE launch: every workgroup computes the same tiles of both
+ * mat-mats against one activation image and applies SiLU * up and the quantizer to them in registers, so the two fp32 [M x N_ff]
+ * intermediates are never written and no separate quantize launch runs (nh_q8_0_gate_up_silu_workspace_bytes == 0 for such a
+ * shape).  Other shapes run nh_q8_0_gemm_tiled twice into `workspace` and nh_q8_0_silu_mul_quantize_tiled.  Either way the bytes are
+ * those of that three-call sequence.  W_gate, W_up: [N_ff x K] tiled; Aq: [M x K] tiled; act: [M x N_ff] tiled; N_ff, K % 128 == 0. */
+int64_t nh_q8_0_gate_up_silu_workspace_bytes(int64_t M, int64_t N_ff, int64_t K);
+int nh_q8_0_gemm_tiled_gate_up_silu(const void* W_gate_tiled, const void* W_up_tiled, const void* Aq_tiled, void* act_tiled_out, void* workspace, int64_t workspace_bytes, int64_t M, int64_t N_ff,
+	int64_t K, void* stream);
+
 /* Fused mul_mat: fp32 activations in, fp32 out -------------------------------------------------- */
 
 /* Scratch the fused call needs for the quantized activations (device bytes, 256-byte aligned by the caller);
@@ -336,6 +348,11 @@ int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void
  *                [5], [6] the grid (column blocks of 128 weight rows, groups of activation strips);
  *   the rest 0.  The same shape under HIP graph capture may take a form without state between launches (no K split). */
 int nh_q8_0_debug_plan_mul_mat(int64_t M, int64_t N, int64_t K, int32_t* host_plan);
+
+/* nh_q8_0_gemm_tiled_gate_up_silu with the fp32 outputs of the two mat-mats copied out as well (gate_out, up_out: [M][N_ff]), so that
+ * the quantized activation can be compared with the CPU quantizer applied to exactly the sums the launch computed. */
+int nh_q8_0_debug_gemm_tiled_gate_up_silu(const void* W_gate_tiled, const void* W_up_tiled, const void* Aq_tiled, void* act_tiled_out, float* gate_out, float* up_out, int64_t M, int64_t N_ff,
+	int64_t K, void* stream);
 
 /* How many polls a workgroup of nh_q8_0_ffn_f32 waits for another workgroup's data before it gives up (default and upper
  * limit 2^20, lower limit 1).  Test hook for the time-out report: with a limit of 1 the down projection's workgroups find

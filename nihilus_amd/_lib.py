@@ -34,6 +34,9 @@ SIGNATURES = {
     "nh_q8_0_get_rows": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "nh_q8_0_get_rows_tiled": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "nh_q8_0_ffn_f32": (_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "nh_q8_0_gate_up_silu_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "nh_q8_0_gemm_tiled_gate_up_silu": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "nh_q8_0_debug_gemm_tiled_gate_up_silu": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "nh_q8_0_decode_layer_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, C.c_float, _i64, _i64, _vp]),
     "nh_q8_0_rms_norm_quantize": (_int, [_vp, _vp, C.c_float, _vp, _i64, _i64, _vp]),
     "nh_q8_0_rms_norm_quantize_tiled": (_int, [_vp, _vp, C.c_float, _vp, _i64, _i64, _vp]),

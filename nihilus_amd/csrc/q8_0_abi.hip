@@ -597,6 +597,48 @@ int nh_q8_0_gemm_tiled_residual(const void* W_tiled, const void* Aq_tiled, const
 	return gemm_common(W_tiled, Aq_tiled, C, M, N, K, true, stream, residual);
 }
 
+int64_t nh_q8_0_gate_up_silu_workspace_bytes(int64_t M, int64_t N_ff, int64_t K) {
+	if (M < 0 || N_ff < 0 || K < 0 || K % nh::GROUP_K != 0 || N_ff % nh::GROUP_K != 0) {
+		return NH_ERR_SHAPE;
+	}
+	if (M == 0 || N_ff == 0 || nh::plan_gate_up_fused(M, N_ff, K)) {
+		return 0;
+	}
+	return 2 * M * N_ff * 4;
+}
+
+static int gate_up_silu_common(const void* W_gate, const void* W_up, const void* Aq, void* act_out, float* gate_out, float* up_out, void* workspace, int64_t workspace_bytes, int64_t M,
+	int64_t N_ff, int64_t K, void* stream) {
+	NH_TRY(check_shape(M, N_ff, K, true));
+	NH_REQUIRE(N_ff % nh::GROUP_K == 0, NH_ERR_SHAPE); // the output is a tiled operand with N_ff as its inner dimension
+	NH_REQUIRE(M <= 65535 * 32, NH_ERR_TOO_LARGE);
+	if (M == 0 || N_ff == 0) {
+		return NH_OK;
+	}
+	NH_REQUIRE(act_out, NH_ERR_NULL_POINTER);
+	NH_REQUIRE(aligned16(act_out) && aligned16(gate_out) && aligned16(up_out) && aligned16(workspace), NH_ERR_ALIGNMENT);
+	if (K > 0) {
+		NH_REQUIRE(W_gate && W_up && Aq, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(W_gate) && aligned16(W_up) && aligned16(Aq), NH_ERR_ALIGNMENT);
+	}
+	const int64_t need = (gate_out && up_out) ? 0 : nh_q8_0_gate_up_silu_workspace_bytes(M, N_ff, K);
+	NH_REQUIRE(workspace_bytes >= need, NH_ERR_ARGUMENT);
+	NH_REQUIRE(need == 0 || workspace, NH_ERR_NULL_POINTER);
+	NH_TRY(require_device());
+	return from_hip(nh::launch_gemm_gate_up_silu(W_gate, W_up, Aq, act_out, gate_out, up_out, static_cast<float*>(workspace), M, N_ff, K, as_stream(stream)));
+}
+
+int nh_q8_0_gemm_tiled_gate_up_silu(const void* W_gate_tiled, const void* W_up_tiled, const void* Aq_tiled, void* act_tiled_out, void* workspace, int64_t workspace_bytes, int64_t M, int64_t N_ff,
+	int64_t K, void* stream) {
+	return gate_up_silu_common(W_gate_tiled, W_up_tiled, Aq_tiled, act_tiled_out, nullptr, nullptr, workspace, workspace_bytes, M, N_ff, K, stream);
+}
+
+int nh_q8_0_debug_gemm_tiled_gate_up_silu(const void* W_gate_tiled, const void* W_up_tiled, const void* Aq_tiled, void* act_tiled_out, float* gate_out, float* up_out, int64_t M, int64_t N_ff,
+	int64_t K, void* stream) {
+	NH_REQUIRE((gate_out && up_out) || M == 0 || N_ff == 0, NH_ERR_NULL_POINTER);
+	return gate_up_silu_common(W_gate_tiled, W_up_tiled, Aq_tiled, act_tiled_out, gate_out, up_out, nullptr, 0, M, N_ff, K, stream);
+}
+
 int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K) {
 	if (M < 0 || K < 0 || K % nh::GROUP_K != 0) {
 		return NH_ERR_SHAPE;

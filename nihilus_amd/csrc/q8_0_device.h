@@ -50,6 +50,15 @@ __device__ __forceinline__ uint16_t load_u16(const uint8_t* p) {
 	return *reinterpret_cast<const uint16_t*>(p);
 }
 
+// q = int8(rne(fl32(f * id))): the last step of quantize_row_q8_0 for one value (reference cpu/avx_2.hpp:4465-4487).
+__device__ __forceinline__ int quantize_value(float f, float id) {
+	const float r = rintf(__fmul_rn(f, id)); // v_rndne_f32: ties to even
+	// x86 cvtps_epi32 yields 0x80000000 for NaN and out-of-range values, which the reference's saturating packs
+	// turn into -128.  Reachable only when 127/amax overflows to inf (amax below ~3.7e-37): inf, and 0*inf = NaN.
+	const int q = (fabsf(r) < 2147483648.0f) ? static_cast<int>(r) : INT32_MIN;
+	return max(-128, min(127, q));
+}
+
 // One lane's share of quantize_row_q8_0 (reference cpu/avx_2.hpp:4439-4489): eight consecutive lanes hold one
 // 32-value block as eight float4.  Returns this lane's four quants packed little-endian; *dh = fp16 bits of d.
 //   amax = max|x_i|; d = fp16_rne(amax / 127.f); id = amax != 0 ? 127.f / amax : 0; q_i = int8(rne(fl32(x_i * id)))
@@ -62,14 +71,7 @@ __device__ __forceinline__ uint32_t quantize_block_lane(float4 v, uint16_t* dh) 
 	const float d  = __fdiv_rn(amax, 127.0f);
 	const float id = (amax != 0.0f) ? __fdiv_rn(127.0f, amax) : 0.0f;
 	*dh			   = float_to_half_bits(d);
-	auto q8		   = [id](float f) -> uint32_t {
-		   const float r = rintf(__fmul_rn(f, id)); // v_rndne_f32: ties to even
-		   // x86 cvtps_epi32 yields 0x80000000 for NaN and out-of-range values, which the reference's saturating packs
-		   // turn into -128.  Reachable only when 127/amax overflows to inf (amax below ~3.7e-37): inf, and 0*inf = NaN.
-		   int q = (fabsf(r) < 2147483648.0f) ? static_cast<int>(r) : INT32_MIN;
-		   q	 = max(-128, min(127, q));
-		   return static_cast<uint32_t>(q) & 0xFFu;
-	};
+	auto q8 = [id](float f) -> uint32_t { return static_cast<uint32_t>(quantize_value(f, id)) & 0xFFu; };
 	return q8(v.x) | (q8(v.y) << 8) | (q8(v.z) << 16) | (q8(v.w) << 24);
 }
 
@@ -305,6 +307,10 @@ inline bool gemv_rows_suits(int64_t M, int64_t N, int64_t K) {
 hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual = nullptr);
 // residual (tiled operands only, or null): C = W . Aq + residual, one fp32 add per element after its sum; may be C itself
 hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s, const float* residual = nullptr);
+// The prefill FFN's first half: act_out (tiled [M x n_ff]) = quantize_row_q8_0(silu(W_gate . Aq) * (W_up . Aq)), one launch where the shape
+// allows it (plan_gate_up_fused in q8_0_plan.h), else two mat-mats into `workspace` (2 * M * n_ff floats) and the SiLU * up quantizer.
+hipError_t launch_gemm_gate_up_silu(const void* w_gate, const void* w_up, const void* aq, void* act_out, float* gate_dbg, float* up_dbg, float* workspace, int64_t M, int64_t n_ff, int64_t K,
+	hipStream_t s);
 // Tiled operands, M <= GEMM_SKINNY_MAX_M (or a tile-kernel grid of at most one workgroup per CU): the streaming MFMA kernel
 // of batched decode (q8_0_gemm_skinny.hip), which walks larger M in groups of 64 rows.
 constexpr int64_t GEMM_SKINNY_MAX_M = 64;

@@ -194,15 +194,30 @@ template<typename T, bool NT> __device__ __forceinline__ T load_sv(gptr_u8 p, ui
 	}
 }
 
-template<int TM, bool DUMP, int KS = 1, bool STREAM = false, bool SPLIT = false>
-__global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* C, const float* R, int32_t* __restrict__ sums, int M, int N,
-	int groups, float* __restrict__ partials = nullptr, unsigned* __restrict__ counters = nullptr) {
+// GATE_UP: the prefill FFN's first half as ONE launch (the reference's mega_ffn composite: ffn_gate and ffn_up mul_mat -> silu ->
+// mul -> activation operand of ffn_down, infra/core_traits.hpp:976-989).  Waves 0, 1 of a workgroup take strips 2 * blockIdx.x + {0, 1}
+// of W (gate), waves 2, 3 the SAME strips of W2 (up), all four against the one activation image in LDS; the loop is the plain
+// kernel's.  Behind it the up waves hand their tiles to the gate waves through LDS, and those apply silu(g) * u and quantize: a
+// 32-value block of the down projection's activation is one activation row against one 32-row weight strip, i.e. one (register,
+// half-wave) of an MFMA result tile -- 32 lanes hold it, its maximum is five cross-lane steps, and the quants go out in the tiled
+// operand layout (through an LDS image of the tile, one 16-byte store per lane).  The two fp32 [M x N] intermediates are never
+// written, the activation is read once for both matrices, and two launches (the second mat-mat and the SiLU * up quantizer) are gone.
+// The arithmetic per value is that of the stand-alone kernels (same fp32 sums, silu_mul, quantize_row_q8_0), so the bytes are theirs.
+// C / C2 (optional, inspection): the fp32 gate / up tiles as the launch computed them.
+template<int TM, bool DUMP, int KS, bool STREAM, bool SPLIT, bool GATE_UP>
+__device__ __forceinline__ void gemm_tiled_body(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* C, const float* R, int32_t* __restrict__ sums, int M, int N, int groups,
+	float* __restrict__ partials, unsigned* __restrict__ counters, const uint8_t* __restrict__ W2, uint8_t* __restrict__ act_out, float* __restrict__ C2) {
 	static_assert(!SPLIT || (KS > 1 && !DUMP), "K over several workgroups continues the K sets' sum");
+	static_assert(!GATE_UP || (KS == 1 && !DUMP && !SPLIT && !STREAM), "the fused gate/up form runs one K set per workgroup");
 	constexpr int DATA_BYTES  = TM * MACRO_BYTES;
 	constexpr int STAGE_BYTES = DATA_BYTES + 16;
 	constexpr int SET_BYTES	   = 2 * STAGE_BYTES + 256; // + 256: where waves that copy no scale table put theirs
 	constexpr int PARK_BYTES   = KS > 1 ? KS * 4 * (KS - 1) * (16 * TM / KS) * 64 * 4 : 0; // the final sum over the K sets, below
-	constexpr int LDS_BYTES	   = KS * SET_BYTES > PARK_BYTES ? KS * SET_BYTES : PARK_BYTES;
+	// GATE_UP epilogue: two up tiles per activation strip as fp32, then per gate wave TM tile images and TM x 32 scales
+	constexpr int XCH_BYTES	   = GATE_UP ? 2 * TM * 16 * 64 * 4 : 0;
+	constexpr int FUSE_BYTES   = GATE_UP ? XCH_BYTES + 2 * TM * (TILE_BYTES + 64) : 0;
+	constexpr int LDS_BASE	   = KS * SET_BYTES > PARK_BYTES ? KS * SET_BYTES : PARK_BYTES;
+	constexpr int LDS_BYTES	   = LDS_BASE > FUSE_BYTES ? LDS_BASE : FUSE_BYTES;
 	__shared__ __align__(16) uint8_t lds_raw[LDS_BYTES];
 	typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 	typedef float v16f __attribute__((ext_vector_type(16)));
@@ -220,7 +235,8 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	const int m_strips = (M + 31) / 32;
 	const int n_strips = (N + 31) / 32;
 	const int ms0	   = blockIdx.y * TM;
-	const int ns	   = blockIdx.x * 4 + wave;
+	const int ns	   = GATE_UP ? blockIdx.x * 2 + (wave & 1) : blockIdx.x * 4 + wave;
+	const uint8_t* Wm  = (GATE_UP && wave >= 2) ? W2 : W; // wave-uniform
 	if ((tid & 255) < 8) {
 		*reinterpret_cast<uint32_t*>(lds + ((tid & 255) >> 2) * STAGE_BYTES + DATA_BYTES + 4 * (tid & 3)) = 0u;
 	}
@@ -273,7 +289,7 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 	};
 	auto fetch_w = [&](int g, w_regs& r) {
 		const int64_t at = w_off + static_cast<int64_t>(g) * MACRO_BYTES;
-		const gptr_u8 p	 = scalar_base(W, at);
+		const gptr_u8 p	 = scalar_base(Wm, at);
 		uint32_t l16 = lane16;
 		asm volatile("" : "+v"(l16));
 		const uint32_t l8 = (l16 & 0x1F0u) >> 1; // the widening of a lane offset has to stay beside its loads for scalar base + 32-bit lane offset to be picked as the addressing mode
@@ -281,7 +297,7 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		for (int k = 0; k < GROUP_BLOCKS; ++k) {
 			r.q[k] = load_sv<v4i, STREAM>(p + k * TILE_BYTES, l16);
 		}
-		r.d = load_sv<v2u, STREAM>(scalar_base(W, at + MACRO_D_OFFSET), l8);
+		r.d = load_sv<v2u, STREAM>(scalar_base(Wm, at + MACRO_D_OFFSET), l8);
 	};
 	// load number p of a group's set (PIECES of them: TM activation tiles, their scale dword, four weight tiles, their scales);
 	// the same loads as fetch_a and fetch_w, which the prologue issues in one go
@@ -295,9 +311,9 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 			ra.d = load_sv<uint32_t, false>(scalar_base(A, sc_off + static_cast<int64_t>(g) * MACRO_BYTES), l16 >> 2);
 		} else if (p < TM + 1 + GROUP_BLOCKS) {
 			const int k = p - TM - 1;
-			rw.q[k] = load_sv<v4i, STREAM>(scalar_base(W, w_off + static_cast<int64_t>(g) * MACRO_BYTES + k * TILE_BYTES), l16);
+			rw.q[k] = load_sv<v4i, STREAM>(scalar_base(Wm, w_off + static_cast<int64_t>(g) * MACRO_BYTES + k * TILE_BYTES), l16);
 		} else {
-			rw.d = load_sv<v2u, STREAM>(scalar_base(W, w_off + static_cast<int64_t>(g) * MACRO_BYTES + MACRO_D_OFFSET), (l16 & 0x1F0u) >> 1);
+			rw.d = load_sv<v2u, STREAM>(scalar_base(Wm, w_off + static_cast<int64_t>(g) * MACRO_BYTES + MACRO_D_OFFSET), (l16 & 0x1F0u) >> 1);
 		}
 	};
 	v16f acc[TM];
@@ -491,6 +507,81 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 		}
 		return;
 	}
+	if constexpr (GATE_UP) {
+		// Every wave is through with the stages (the last trip ended in a barrier).  The gate wave and the up wave of a strip share
+		// the work behind the loop: registers 0..7 of every tile are finished by the gate wave, 8..15 by the up wave, each handing
+		// the other the half it does not finish (the exp and the divides of SiLU and of the quantizer are a quarter of the loop's
+		// VALU work; on two of the four waves alone they cost the launch 6 %).
+		const int pair	 = wave & 1;
+		const bool is_up = wave >= 2;
+		float* xch		 = reinterpret_cast<float*>(lds_raw); // [pair][TM][16][64]: slot (i, e) holds the value of the wave that does not finish it
+#pragma unroll
+		for (int i = 0; i < TM; ++i) {
+#pragma unroll
+			for (int e = 0; e < 8; ++e) {
+				const int give						  = is_up ? e : e + 8;
+				xch[((pair * TM + i) * 16 + give) * 64 + lane] = acc[i][give];
+			}
+		}
+		float* dbg = is_up ? C2 : C; // inspection copies of the fp32 tiles
+		if (dbg) {
+			const int n = ns * 32 + (lane & 31);
+#pragma unroll
+			for (int i = 0; i < TM; ++i) {
+#pragma unroll
+				for (int e = 0; e < 16; ++e) {
+					const int m = (ms0 + i) * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+					if (m < M && n < N) {
+						dbg[static_cast<int64_t>(m) * N + n] = acc[i][e];
+					}
+				}
+			}
+		}
+		__syncthreads();
+		uint8_t* image = lds_raw + XCH_BYTES + pair * TM * (TILE_BYTES + 64); // the pair's TM tile images, each followed by its 32 scales
+		const int j	   = lane & 31; // the lane's weight row = quant j of the block
+#pragma unroll
+		for (int i = 0; i < TM; ++i) {
+			uint8_t* tile	 = image + i * (TILE_BYTES + 64);
+			uint16_t* scales = reinterpret_cast<uint16_t*>(tile + TILE_BYTES);
+#pragma unroll
+			for (int e8 = 0; e8 < 8; ++e8) {
+				const int e		  = is_up ? e8 + 8 : e8;
+				const float other = xch[((pair * TM + i) * 16 + e) * 64 + lane];
+				const float v	  = is_up ? silu_mul(other, acc[i][e]) : silu_mul(acc[i][e], other);
+				// the block = this register over the 32 lanes of the half-wave: quantize_row_q8_0 on it
+				float amax = fabsf(v);
+#pragma unroll
+				for (int off = 16; off >= 1; off >>= 1) {
+					amax = fmaxf(amax, __shfl_xor(amax, off));
+				}
+				const float d  = __fdiv_rn(amax, 127.0f);
+				const float id = (amax != 0.0f) ? __fdiv_rn(127.0f, amax) : 0.0f;
+				const int r	   = 8 * (e >> 2) + 4 * half + (e & 3); // row within the activation strip
+				tile[16 * (r + 32 * (j >> 4)) + (j & 15)] = static_cast<uint8_t>(quantize_value(v, id));
+				if (j == 0) {
+					scales[r] = float_to_half_bits(d);
+				}
+			}
+		}
+		__syncthreads(); // both waves of a pair have filled its images
+		// tile i of the pair goes out through the gate wave (even i) or the up wave (odd i): one 16-byte store per lane
+		const int out_groups = N / GROUP_K; // the activation is [M x N]: N / 128 groups per strip, this strip's block is ns
+		if (ns < n_strips) {
+#pragma unroll
+			for (int i = 0; i < TM; ++i) {
+				if ((i & 1) == (is_up ? 1 : 0) && ms0 + i < m_strips) {
+					const uint8_t* tile = image + i * (TILE_BYTES + 64);
+					uint8_t* macro		= act_out + macro_offset(ms0 + i, ns / GROUP_BLOCKS, out_groups);
+					*reinterpret_cast<v4i*>(macro + (ns % GROUP_BLOCKS) * TILE_BYTES + 16 * lane) = *reinterpret_cast<const v4i*>(tile + 16 * lane);
+					if (lane < STRIP_ROWS) {
+						*reinterpret_cast<uint16_t*>(macro + MACRO_D_OFFSET + 8 * lane + 2 * (ns % GROUP_BLOCKS)) = reinterpret_cast<const uint16_t*>(tile + TILE_BYTES)[lane];
+					}
+				}
+			}
+		}
+		return;
+	}
 	if constexpr (!DUMP) {
 		const int n = ns * 32 + (lane & 31);
 #pragma unroll
@@ -505,6 +596,19 @@ __global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* 
 			}
 		}
 	}
+}
+
+template<int TM, bool DUMP, int KS = 1, bool STREAM = false, bool SPLIT = false>
+__global__ __launch_bounds__(256 * KS, 4) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const uint8_t* __restrict__ A, float* C, const float* R, int32_t* __restrict__ sums, int M, int N,
+	int groups, float* __restrict__ partials, unsigned* __restrict__ counters) {
+	gemm_tiled_body<TM, DUMP, KS, STREAM, SPLIT, false>(W, A, C, R, sums, M, N, groups, partials, counters, nullptr, nullptr, nullptr);
+}
+
+// the fused gate / up form (GATE_UP above): N = rows of each of the two matrices; gate_out / up_out optional
+template<int TM>
+__global__ __launch_bounds__(256, 4) void gemm_gate_up_kernel(const uint8_t* __restrict__ W_gate, const uint8_t* __restrict__ W_up, const uint8_t* __restrict__ A, uint8_t* __restrict__ act_out,
+	float* __restrict__ gate_out, float* __restrict__ up_out, int M, int N, int groups) {
+	gemm_tiled_body<TM, false, 1, false, false, true>(W_gate, A, gate_out, nullptr, nullptr, M, N, groups, nullptr, nullptr, W_up, act_out, up_out);
 }
 
 // Executes a cut made by plan_gemm_tile (q8_0_plan.h): TM activation strips per wave, KS sets of four waves per workgroup,
@@ -544,6 +648,39 @@ static hipError_t launch_gemm_tiled(const gemm_tile_cut& cut, const uint8_t* w, 
 		return cut.tm == 2 ? launch_gemm_tiled_t<2, true>(cut, w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, true>(cut, w, a, C, R, sums, m, n, k, s);
 	}
 	return cut.tm == 2 ? launch_gemm_tiled_t<2, false>(cut, w, a, C, R, sums, m, n, k, s) : launch_gemm_tiled_t<1, false>(cut, w, a, C, R, sums, m, n, k, s);
+}
+
+// act_out (tiled, [M x n_ff]) = quantize_row_q8_0(silu(W_gate . Aq) * (W_up . Aq)); gate_dbg / up_dbg: optional fp32 copies of the two
+// mat-mats' outputs.  workspace: 2 * M * n_ff floats for shapes the fused form does not take (plan_gate_up_fused), else unused.
+hipError_t launch_gemm_gate_up_silu(const void* w_gate, const void* w_up, const void* aq, void* act_out, float* gate_dbg, float* up_dbg, float* workspace, int64_t M, int64_t n_ff, int64_t K,
+	hipStream_t s) {
+	if (M == 0 || n_ff == 0) {
+		return hipSuccess;
+	}
+	gemm_tile_cut cut{};
+	if (plan_gate_up_fused(M, n_ff, K, &cut)) {
+		const uint8_t* wg = static_cast<const uint8_t*>(w_gate);
+		const uint8_t* wu = static_cast<const uint8_t*>(w_up);
+		const uint8_t* a  = static_cast<const uint8_t*>(aq);
+		uint8_t* out	  = static_cast<uint8_t*>(act_out);
+		const int m = static_cast<int>(M), n = static_cast<int>(n_ff), groups = static_cast<int>(K / GROUP_K);
+		const dim3 grid(cut.grid_x, cut.grid_y);
+		if (cut.tm == 2) {
+			return launch_kernel(KIND_GEMM, gemm_gate_up_kernel<2>, grid, dim3(256), 0, s, wg, wu, a, out, gate_dbg, up_dbg, m, n, groups);
+		}
+		return launch_kernel(KIND_GEMM, gemm_gate_up_kernel<1>, grid, dim3(256), 0, s, wg, wu, a, out, gate_dbg, up_dbg, m, n, groups);
+	}
+	float* gate = gate_dbg ? gate_dbg : workspace;
+	float* up	= up_dbg ? up_dbg : workspace + M * n_ff;
+	hipError_t e = launch_gemm(w_gate, aq, gate, nullptr, M, n_ff, K, true, s);
+	if (e != hipSuccess) {
+		return e;
+	}
+	e = launch_gemm(w_up, aq, up, nullptr, M, n_ff, K, true, s);
+	if (e != hipSuccess) {
+		return e;
+	}
+	return launch_silu_mul_quantize(gate, up, act_out, M, n_ff, true, s);
 }
 
 __global__ void zero_c_kernel(float* c, const float* src, int64_t n) {

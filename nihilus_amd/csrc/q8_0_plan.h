@@ -137,6 +137,26 @@ inline gemm_plan plan_gemm(int64_t M, int64_t N, int64_t K) {
 	return p;
 }
 
+// The prefill FFN's gate and up mat-mats with SiLU * up and the quantizer behind them: one launch of the tile kernel's fused form
+// where each matrix alone would take the prefill tile kernel and the doubled grid runs one K set per workgroup; otherwise the two
+// mat-mats and the quantizer as launches of their own (through an fp32 workspace).
+inline bool plan_gate_up_fused(int64_t M, int64_t n_ff, int64_t K, gemm_tile_cut* cut = nullptr) {
+	if (M <= 0 || n_ff <= 0 || K <= 0 || n_ff % GROUP_K != 0 || K % GROUP_K != 0) {
+		return false;
+	}
+	if (plan_gemm(M, n_ff, K).kernel != MM_GEMM_TILE) {
+		return false;
+	}
+	const gemm_tile_cut c = plan_gemm_tile(M, 2 * n_ff, K, false); // grid_x = n_ff / 64 workgroups of two gate and two up strips
+	if (c.ks != 1) {
+		return false;
+	}
+	if (cut) {
+		*cut = c;
+	}
+	return true;
+}
+
 // nh_q8_0_mul_mat: fp32 activations [M][K] against a tiled weight [N][K].
 struct mul_mat_plan {
 	int kernel; // mul_mat_kernel

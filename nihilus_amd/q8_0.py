@@ -300,6 +300,24 @@ def gemm_residual(w_tiled: torch.Tensor, aq_tiled: torch.Tensor, residual: torch
     return c
 
 
+def gate_up_silu(w_gate: torch.Tensor, w_up: torch.Tensor, aq_tiled: torch.Tensor, m: int, n_ff: int, k: int, debug: bool = False):
+    """Tiled Q8_0 activation of the down projection: quantize(silu(W_gate . Aq) * (W_up . Aq)) (nh_q8_0_gemm_tiled_gate_up_silu).
+    debug=True also returns the fp32 gate and up outputs the call computed."""
+    lib = _lib.lib()
+    out = torch.empty(tiled_bytes(m, n_ff), dtype=torch.uint8, device=aq_tiled.device)
+    if debug:
+        gate = torch.empty((m, n_ff), dtype=torch.float32, device=aq_tiled.device)
+        up = torch.empty((m, n_ff), dtype=torch.float32, device=aq_tiled.device)
+        _lib.check("nh_q8_0_debug_gemm_tiled_gate_up_silu", lib.nh_q8_0_debug_gemm_tiled_gate_up_silu(w_gate.data_ptr(), w_up.data_ptr(), aq_tiled.data_ptr(), out.data_ptr(), gate.data_ptr(),
+                                                                                                          up.data_ptr(), m, n_ff, k, _stream()))
+        return out, gate, up
+    need = lib.nh_q8_0_gate_up_silu_workspace_bytes(m, n_ff, k)
+    _lib.check("nh_q8_0_gate_up_silu_workspace_bytes", need if need < 0 else 0)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=aq_tiled.device)
+    _lib.check("nh_q8_0_gemm_tiled_gate_up_silu", lib.nh_q8_0_gemm_tiled_gate_up_silu(w_gate.data_ptr(), w_up.data_ptr(), aq_tiled.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), m, n_ff, k, _stream()))
+    return out
+
+
 def mul_mat(w_tiled: torch.Tensor, x: torch.Tensor, n: int, k: int, workspace: torch.Tensor | None = None, residual: torch.Tensor | None = None) -> torch.Tensor:
     """fp32 activations [M, K] x tiled Q8_0 weight [N, K] -> fp32 [M, N]: quantize + GEMV/GEMM (+ residual [M, N] if given)."""
     w_tiled, x = _dev(w_tiled, torch.uint8, "w_tiled"), _dev(x, torch.float32, "x")
