@@ -387,6 +387,10 @@ __device__ __forceinline__ float gemv_chunk(const uint8_t* __restrict__ w_strip,
 		NH_CHUNK_CASE(2)
 		NH_CHUNK_CASE(3)
 		NH_CHUNK_CASE(4)
+		NH_CHUNK_CASE(5)
+		NH_CHUNK_CASE(6)
+		NH_CHUNK_CASE(7)
+		NH_CHUNK_CASE(8)
 		default:
 			break;
 	}

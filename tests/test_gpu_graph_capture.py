@@ -64,6 +64,50 @@ def test_captured_launches_replay_with_new_inputs(q8, oracle):
     assert rel_l2(got[0], oracle.gemv(to_host(q8.untile(w, n, k)), aq, n, k)) <= REL_L2_TOL
 
 
+def test_captured_decode_layer_replays_with_new_inputs(q8, oracle):
+    # the chained decode layer hands data between its stages under a per-launch epoch: a capturing stream gets the three launches it
+    # stands for (themselves in their replay-safe forms); replays must follow new inputs and agree with the eager one-launch form
+    import torch
+
+    from nihilus_amd import _lib
+
+    _lib.check("nh_q8_0_prepare", _lib.lib().nh_q8_0_prepare())
+    rng = np.random.default_rng(23)
+    n_embd, n_ff, nxt = 1024, 3584, [1024, 256]
+    sig = lambda k_in: 1.0 / (58.0 * np.sqrt(k_in))  # noqa: E731
+    ws = {name: q8.tile(to_dev(random_blocks(rng, n, k, sig(k))), n, k) for name, n, k in
+          [("o", n_embd, n_embd), ("g", n_ff, n_embd), ("u", n_ff, n_embd), ("d", n_embd, n_ff), ("q", 1024, n_embd), ("k", 256, n_embd)]}
+    norm1 = to_dev((1.0 + 0.1 * rng.standard_normal(n_embd)).astype(np.float32))
+    norm2 = to_dev((1.0 + 0.1 * rng.standard_normal(n_embd)).astype(np.float32))
+    attn = torch.zeros(n_embd, dtype=torch.float32, device="cuda")
+    x = torch.zeros(n_embd, dtype=torch.float32, device="cuda")
+
+    def launch():
+        h, y, outs = q8.decode_layer(ws["o"], attn, x, ws["g"], ws["u"], ws["d"], norm1, [ws["q"], ws["k"]], nxt, norm2, 1e-5, n_embd, n_ff)
+        return [h, y, *outs]
+
+    def new_inputs(seed):
+        attn.copy_(to_dev(oracle.fill_activations(seed, n_embd)))
+        x.copy_(to_dev(oracle.fill_activations(seed + 500, n_embd)))
+
+    new_inputs(1)
+    launch()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = launch()
+    for seed in (2, 3, 4):
+        new_inputs(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [to_host(t).copy() for t in captured]
+        want = [to_host(t) for t in launch()]  # eager: one launch, fresh epoch, between the replays
+        torch.cuda.synchronize()
+        assert rel_l2(got[0], want[0]) < 2e-6, seed  # attn_out + residual: same arithmetic, another cut
+        for g, e in zip(got[1:], want[1:]):
+            assert np.isfinite(g).all() and rel_l2(g, e) <= 2e-3, seed  # quantizers sit between the stages
+
+
 def test_captured_batch_of_independent_mat_vecs(q8, oracle):
     # a batch call whose entries the runner may group: under capture the short-K ones still share a launch (no per-launch
     # state when K is not split), the long-K one falls back to its own unsplit launch; replays must follow new inputs
