@@ -46,6 +46,8 @@ SHAPES = [
     (2048, 5632, (), False),  # nothing behind the block
     (8192, 28672, (8192, 1024, 1024), True),  # LLaMA-3-70B block: whole attn_out strips in the separate launch too, so the same cuts everywhere
     (8192, 3584, (1024, 256), False),  # the longest hidden state the one launch takes: four groups per wave, gate/up waves take one matrix each
+    (4096, 9216, (8000,), False),  # a row-cut down stage with a long, ragged stage behind it
+    (4096, 14336, (1024,), False),  # ... and with a short one
 ]
 
 
