@@ -285,7 +285,8 @@ def main() -> int:
         torch.cuda.empty_cache()
         l70 = side_workload("llama70b", 100, 10)
         result["llama70b"] = {"workload": l70["config"]["workload"], "unit": "us per nh_q8_0_mul_mat call; pct_hbm = weight bytes / time against 8 TB/s",
-                              "rows": [{k: r[k] for k in ("projection", "M", "N", "K", "us", "kernel", "pct_hbm")} for r in l70["rows"]]}
+                              "rows": [{k: r[k] for k in ("projection", "M", "N", "K", "us", "kernel", "pct_hbm")} for r in l70["rows"]],
+                              "decode_block": l70["decode_block"]}
         torch.cuda.empty_cache()
         probe = machine_probe("coissue_probe")
         if probe is not None:
@@ -627,7 +628,52 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
                              "pct_hbm": round(100 * wbytes / sec / 1e9 / HBM_PEAK_GBS, 1), "TOPs": round(2.0 * m * n * k / sec / 1e12, 2)})
             del ws
             torch.cuda.empty_cache()
+        # one 70B block's decode mat-vecs from one attention to the next (attn_out + residual -> norm -> gate/up -> SiLU*up -> down +
+        # residual -> norm -> the next block's q/k/v), batch 1: as one launch and as the three launches it stands for; two weight sets
+        # (910 MB each) rotated
+        import ctypes as C
+        e70, f70, kv70 = 8192, 28672, 1024
+        shapes70 = ((e70, e70), (f70, e70), (f70, e70), (e70, f70), (e70, e70), (kv70, e70), (kv70, e70))  # o, gate, up, down, next q, k, v
+        blocks70 = [[q8_0.tile(q8_0.fill_weight_blocks(31 + 7 * c_i + j, n, k), n, k) for j, (n, k) in enumerate(shapes70)] for c_i in range(2)]
+        block_bytes = sum(n * (k // 32) * 34 for n, k in shapes70)
+        attn70, in70 = q8_0.fill_activations(3, e70), q8_0.fill_activations(4, e70)
+        ones70 = torch.ones(e70, dtype=torch.float32, device=attn70.device)
+        h70, l70o = torch.empty_like(attn70), torch.empty_like(attn70)
+        y70 = [torch.empty(n, dtype=torch.float32, device=attn70.device) for n in (e70, kv70, kv70)]
+        vp3, i3 = C.c_void_p * 3, C.c_int64 * 3
+        yp, np3 = vp3(*[t.data_ptr() for t in y70]), i3(e70, kv70, kv70)
+        wp = [vp3(*[t.data_ptr() for t in b[4:7]]) for b in blocks70]
+        eps70 = C.c_float(1e-5)
+        it70 = [0]
+
+        def one_launch():
+            b = blocks70[it70[0] % 2]
+            it70[0] += 1
+            _lib.check("nh_q8_0_decode_layer_f32", lib.nh_q8_0_decode_layer_f32(b[0].data_ptr(), attn70.data_ptr(), in70.data_ptr(), h70.data_ptr(), b[1].data_ptr(), b[2].data_ptr(), b[3].data_ptr(),
+                                                                            ones70.data_ptr(), l70o.data_ptr(), wp[(it70[0] - 1) % 2], yp, np3, 3, ones70.data_ptr(), eps70, e70, f70, stream))
+
+        def three_launches():
+            b = blocks70[it70[0] % 2]
+            it70[0] += 1
+            _lib.check("o", lib.nh_q8_0_gemv_tiled_residual_f32(b[0].data_ptr(), attn70.data_ptr(), in70.data_ptr(), h70.data_ptr(), e70, e70, stream))
+            _lib.check("ffn", lib.nh_q8_0_ffn_f32(b[1].data_ptr(), b[2].data_ptr(), b[3].data_ptr(), h70.data_ptr(), ones70.data_ptr(), eps70, h70.data_ptr(), l70o.data_ptr(), f70, e70, e70, stream))
+            _lib.check("qkv", lib.nh_q8_0_gemv_tiled_multi_norm_f32(wp[(it70[0] - 1) % 2], yp, np3, 3, l70o.data_ptr(), ones70.data_ptr(), eps70, e70, stream))
+
+        block = {"bytes": block_bytes}
+        for name, fn in (("one_launch", one_launch), ("three_launches", three_launches)):
+            warm_up(fn, 0.0)
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            sec = (time.perf_counter() - t0) / steps
+            block[name + "_us"] = round(sec * 1e6, 2)
+            block[name + "_pct_hbm"] = round(100 * block_bytes / sec / 1e9 / HBM_PEAK_GBS, 1)
+        block["outputs_finite"] = bool(torch.isfinite(y70[0]).all().item() and torch.isfinite(l70o).all().item())
+        del blocks70
+        torch.cuda.empty_cache()
         return {"metric": "Q8_0 mul_mat weight-streaming GB/s at LLaMA-3-70B projection shapes, batched decode", "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+                "decode_block": block,
                 "higher_is_better": True, "dtype": "int8 x int8 -> int32 block sums, fp32 scale-accumulate", "data": "synthetic",
                 "config": {"workload": "nh_q8_0_mul_mat, fp32 activations [M x K] x Q8_0 W at the 70B shapes, M in {1, 4, 16, 64}, activation quantize included, "
                            "weight sets rotated over > 1 GB (lm_head: one 1.1 GB matrix)"}, "rows": rows}
