@@ -631,7 +631,6 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
         # one 70B block's decode mat-vecs from one attention to the next (attn_out + residual -> norm -> gate/up -> SiLU*up -> down +
         # residual -> norm -> the next block's q/k/v), batch 1: as one launch and as the three launches it stands for; two weight sets
         # (910 MB each) rotated
-        import ctypes as C
         e70, f70, kv70 = 8192, 28672, 1024
         shapes70 = ((e70, e70), (f70, e70), (f70, e70), (e70, f70), (e70, e70), (kv70, e70), (kv70, e70))  # o, gate, up, down, next q, k, v
         blocks70 = [[q8_0.tile(q8_0.fill_weight_blocks(31 + 7 * c_i + j, n, k), n, k) for j, (n, k) in enumerate(shapes70)] for c_i in range(2)]

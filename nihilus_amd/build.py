@@ -12,7 +12,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_NAME = "libnihilus_q8_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-SOURCES = ["q8_0_abi.hip", "q8_0_quantize.hip", "q8_0_layout.hip", "q8_0_get_rows.hip", "q8_0_gemv.hip", "q8_0_gemv_rows.hip", "q8_0_gemv_group.hip", "q8_0_mul_mat_f32act.hip", "q8_0_ffn.hip", "q8_0_decode_layer.hip", "q8_0_gemm.hip", "q8_0_gemm_skinny.hip", "q8_0_profile.hip", "gguf_q8_0.cpp"]
+SOURCES = ["q8_0_abi.hip", "q8_0_quantize.hip", "q8_0_layout.hip", "q8_0_get_rows.hip", "q8_0_gemv.hip", "q8_0_gemv_rows.hip", "q8_0_gemv_rows_mfma.hip", "q8_0_gemv_group.hip", "q8_0_mul_mat_f32act.hip", "q8_0_ffn.hip", "q8_0_decode_layer.hip", "q8_0_gemm.hip", "q8_0_gemm_skinny.hip", "q8_0_profile.hip", "gguf_q8_0.cpp"]
 
 # -packed-fp32-ops off: v_pk_{add,mul,fma}_f32 are kept out of the generated code on purpose.
 # No -ffast-math: the quantizer needs IEEE divide, unfused multiply and round-half-even.

@@ -664,6 +664,12 @@ static int mul_mat_common(const void* W_tiled, const float* x, const float* resi
 	if (M == 1) { // quantize fused into the mat-vec: the workspace stays unused
 		return residual ? nh_q8_0_gemv_tiled_residual_f32(W_tiled, x, residual, y, N, K, stream) : nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream);
 	}
+	if (plan.kernel == nh::MM_GEMV_ROWS_MFMA) { // up to eight rows: the streaming kernel with the rows as an MFMA operand
+		NH_REQUIRE(W_tiled && y, NH_ERR_NULL_POINTER);
+		NH_REQUIRE(aligned16(W_tiled) && aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
+		NH_TRY(require_device());
+		return from_hip(nh::launch_gemv_rows_mfma(W_tiled, x, y, M, N, K, as_stream(stream), residual));
+	}
 	if (plan.kernel == nh::MM_GEMV_ROWS) { // a few rows: the same streaming kernel with M dot products per weight tile
 		NH_REQUIRE(W_tiled && y, NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(W_tiled) && aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
@@ -685,6 +691,7 @@ int nh_q8_0_debug_plan_mul_mat(int64_t M, int64_t N, int64_t K, int32_t* host_pl
 	host_plan[1] = p.quantize_launch;
 	switch (p.kernel) {
 		case nh::MM_GEMV:
+		case nh::MM_GEMV_ROWS_MFMA:
 			host_plan[2] = p.gemv.splits;
 			host_plan[3] = p.gemv.tiles;
 			host_plan[4] = p.gemv_row_parts;

@@ -299,12 +299,12 @@ hipError_t launch_gemv_independent(const gemv_group_op* ops, int64_t count, hipS
 // 2 <= M <= GEMV_ROWS_MAX fp32 activation rows against one tiled weight matrix: the streaming mat-vec with M dot products per
 // weight tile, quantize included (q8_0_gemv_rows.hip).  y is [M][N].
 constexpr int64_t GEMV_ROWS_MAX = 3;
-constexpr int64_t GEMV_ROWS_WIDE_MAX = 5; // what the kernel takes; above GEMV_ROWS_MAX only for small matrices (gemv_rows_suits)
-// whether M rows against an N x K matrix are better served by this kernel than by quantize + the MFMA streaming kernel
-inline bool gemv_rows_suits(int64_t M, int64_t N, int64_t K) {
-	return M >= 2 && (M <= GEMV_ROWS_MAX || (M <= GEMV_ROWS_WIDE_MAX && N * (K / QK) * BLOCK_BYTES <= (int64_t{ 40 } << 20)));
+inline bool gemv_rows_suits(int64_t M, int64_t /*N*/, int64_t /*K*/) {
+	return M >= 2 && M <= GEMV_ROWS_MAX;
 }
 hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual = nullptr);
+// 1 <= M <= 8 rows on the matrix cores, quantize included, no workspace (q8_0_gemv_rows_mfma.hip).  y is [M][N].
+hipError_t launch_gemv_rows_mfma(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual = nullptr);
 // residual (tiled operands only, or null): C = W . Aq + residual, one fp32 add per element after its sum; may be C itself
 hipError_t launch_gemm(const void* W, const void* Aq, float* C, int32_t* sums, int64_t M, int64_t N, int64_t K, bool tiled, hipStream_t s, const float* residual = nullptr);
 // The prefill FFN's first half: act_out (tiled [M x n_ff]) = quantize_row_q8_0(silu(W_gate . Aq) * (W_up . Aq)), one launch where the shape

@@ -1,4 +1,4 @@
-// Batched decode with a handful of activation rows (2 <= M <= GEMV_ROWS_WIDE_MAX): y[m][n] = dot(W row n, quantize(x row m)), gfx950.
+// Batched decode with two or three activation rows (2 <= M <= GEMV_ROWS_MAX): y[m][n] = dot(W row n, quantize(x row m)), gfx950.
 //
 // The streaming mat-vec again (q8_0_gemv.hip): one workgroup of sixteen waves per (32-row weight strip, K split), every
 // wave puts all the weight loads of its K range in flight before it waits for anything, the activation slice is quantized
@@ -7,11 +7,10 @@
 // instead of one and runs MR dot products against every weight tile it fetched, so the weights are still read exactly
 // once and no quantize launch, no quantized copy of the activations and no 32-row MFMA tile (30 of whose rows would be
 // padding at M = 2) is involved.  The integer dots and the quantizer cost MR times those of the mat-vec (every strip's
-// workgroup quantizes the rows again), which an HBM-bound kernel can afford for two or three rows; from four on the MFMA
-// streaming kernel (q8_0_gemm_skinny.hip), whose cost does not grow with M up to 32, measured faster -- except on small
-// matrices with four or five rows, where the quantize launch that the MFMA kernel needs in front of it costs more than the
-// extra dot products do ([4096 x 4096], M = 4: 8.0 us against 9.2-12.4 us for quantize + MFMA kernel, depending on the host's
-// launch rate; at eight rows the two meet, and on a 60 MB matrix the MFMA kernel wins from four).
+// workgroup quantizes the rows again), which an HBM-bound kernel can afford for two or three rows.  From four rows on every lane's
+// LDS reads of the rows' quants (one 16-byte read per lane, block and row) are what a CU waits for ([4096 x 4096]: 4.6 us at two
+// rows, 8.1 us at four): there the rows go to the matrix cores instead (q8_0_gemv_rows_mfma.hip on small matrices, the quantize
+// launch and the MFMA kernels otherwise).
 // Arithmetic per output element: exact int32 block sums, fp32 scale-and-accumulate in the mat-vec's fixed order
 // (reference vec_dot_q8_0_q8_0, cpu/avx_2.hpp:4534-4747); output [M][N] with n fastest (cpu/avx_2.hpp:4934).
 #include "q8_0_gemv_tiled.h"
@@ -190,8 +189,8 @@ template<int MR> static hipError_t launch_rows_m(const gemv_plan& p, const uint8
 
 hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, int64_t N, int64_t K, hipStream_t s, const float* residual) {
 	const int64_t strips = (N + STRIP_ROWS - 1) / STRIP_ROWS;
-	if (strips == 0 || M < 2 || M > GEMV_ROWS_WIDE_MAX) {
-		return M < 2 || M > GEMV_ROWS_WIDE_MAX ? hipErrorInvalidValue : hipSuccess;
+	if (strips == 0 || M < 2 || M > GEMV_ROWS_MAX) {
+		return M < 2 || M > GEMV_ROWS_MAX ? hipErrorInvalidValue : hipSuccess;
 	}
 	// K is cut until a wave owns at most two groups (the register budget above); the split scratch holds one unit per
 	// (strip, activation row, split)
@@ -221,16 +220,7 @@ hipError_t launch_gemv_rows(const void* W, const float* x, float* y, int64_t M, 
 	}
 	const uint8_t* w = static_cast<const uint8_t*>(W);
 	const int n		 = static_cast<int>(N);
-	switch (M) {
-		case 2:
-			return launch_rows_m<2>(p, w, x, y, residual, n, sc, s);
-		case 3:
-			return launch_rows_m<3>(p, w, x, y, residual, n, sc, s);
-		case 4:
-			return launch_rows_m<4>(p, w, x, y, residual, n, sc, s);
-		default:
-			return launch_rows_m<5>(p, w, x, y, residual, n, sc, s);
-	}
+	return M == 2 ? launch_rows_m<2>(p, w, x, y, residual, n, sc, s) : launch_rows_m<3>(p, w, x, y, residual, n, sc, s);
 }
 
 } // namespace nh

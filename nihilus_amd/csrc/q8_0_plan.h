@@ -13,10 +13,11 @@ namespace nh {
 enum mul_mat_kernel : int {
 	MM_NOTHING			= 0, // an empty problem: nothing, or a fill of the output
 	MM_GEMV				= 1, // M == 1: quantize inside the streaming mat-vec (gemv_tiled_kernel)
-	MM_GEMV_ROWS		= 2, // 2..5 rows: the streaming mat-vec with one dot product per row (gemv_rows_kernel), quantize inside
+	MM_GEMV_ROWS		= 2, // 2, 3 rows: the streaming mat-vec with one dot product per row (gemv_rows_kernel), quantize inside
 	MM_GEMM_SKINNY		= 3, // quantize launch + weight-streaming MFMA kernel (gemm_skinny_kernel)
 	MM_GEMM_TILE_STREAM = 4, // quantize launch + MFMA tile kernel with non-temporal weight loads (batched decode on large matrices)
 	MM_GEMM_TILE		= 5, // quantize launch + MFMA tile kernel (prefill)
+	MM_GEMV_ROWS_MFMA	= 6, // 4..8 rows on small matrices: the streaming mat-vec with the rows as an MFMA operand (gemv_rows8_kernel), quantize inside
 };
 
 constexpr int SK_WAVES			  = 8; // waves per workgroup of the weight-streaming MFMA kernel
@@ -157,6 +158,45 @@ inline bool plan_gate_up_fused(int64_t M, int64_t n_ff, int64_t K, gemm_tile_cut
 	return true;
 }
 
+// The eight-row MFMA mat-vec's cut (q8_0_gemv_rows_mfma.hip): K over workgroups until a wave owns at most two groups (its
+// register budget), within the split scratch's units (one per strip, activation row and split); matrices with few strips are cut
+// further so that the launch reaches the CUs.  Under HIP graph capture: no K split (a replay could not renew the hand-off's epoch),
+// a chunked walk instead.
+constexpr int GEMV_ROWS_MFMA_MAX = 8;
+// Where it is the fastest form (measured against what ran before, quantize launch included; us):
+//   [4096 x 4096]   17.8 MB   M = 4:  6.0 against  8.1 (dot-product kernel)      M = 8:  7.5 against 12.2 (quantize + streaming MFMA kernel)
+//   [1024 x 8192]    8.9 MB   M = 4:  6.0 against  7.3
+//   [14336 x 4096]  62.4 MB   M = 4: 14.5 against 15.6                            M = 8: 19.3 against 15.7
+//   [8192 x 8192]   71.3 MB   M = 4: 18.4 against 21.2
+//   [28672 x 8192]   250 MB   M = 4: 51   against 43.6;  [128256 x 8192]: 199 against 167
+// Every strip's workgroup quantizes all the rows again, which costs in proportion to M and to the matrix: up to eight rows on
+// matrices of at most 40 MB, four on matrices of at most 80 MB.  (Two and three rows stay on the dot-product kernel.)
+inline bool gemv_rows_mfma_suits(int64_t M, int64_t N, int64_t K) {
+	const int64_t weight_bytes = N * (K / QK) * BLOCK_BYTES;
+	return M >= 4 && M <= GEMV_ROWS_MFMA_MAX && (weight_bytes <= (int64_t{ 40 } << 20) || (M == 4 && weight_bytes <= (int64_t{ 80 } << 20)));
+}
+inline gemv_plan plan_gemv_rows_mfma(int64_t strips, int64_t K, bool capturing) {
+	gemv_plan p;
+	p.strips	   = static_cast<int>(strips);
+	p.groups	   = static_cast<int>(K / GROUP_K);
+	p.splits	   = 1;
+	auto tiles_for = [&](int sp) { return (p.groups + GEMV_WAVES * sp - 1) / (GEMV_WAVES * sp); };
+	auto room	   = [&](int sp) { return strips * GEMV_ROWS_MFMA_MAX * sp <= GEMV_MAX_SPLIT_UNITS; };
+	while (tiles_for(p.splits) > 2 && room(p.splits * 2)) {
+		p.splits *= 2;
+	}
+	// (a workgroup per CU, not per two as in the dot-product kernel: every workgroup quantizes its K range of all the rows, and that
+	// work is what the launch waits for -- [4096 x 4096] at 8 rows: 9.8 us with 128 workgroups, 7.5 us with 256)
+	while (strips * p.splits < 256 && tiles_for(p.splits) > 1 && room(p.splits * 2)) {
+		p.splits *= 2;
+	}
+	if (capturing) {
+		p.splits = 1;
+	}
+	p.tiles = tiles_for(p.splits);
+	return p;
+}
+
 // nh_q8_0_mul_mat: fp32 activations [M][K] against a tiled weight [N][K].
 struct mul_mat_plan {
 	int kernel; // mul_mat_kernel
@@ -184,6 +224,12 @@ inline mul_mat_plan plan_mul_mat(int64_t M, int64_t N, int64_t K) {
 		p.kernel		 = MM_GEMV;
 		p.gemv			 = plan_gemv((N + STRIP_ROWS - 1) / STRIP_ROWS, K);
 		p.gemv_row_parts = plan_gemv_row_parts(p.gemv);
+		return p;
+	}
+	if (gemv_rows_mfma_suits(M, N, K)) {
+		p.kernel		 = MM_GEMV_ROWS_MFMA;
+		p.gemv			 = plan_gemv_rows_mfma((N + STRIP_ROWS - 1) / STRIP_ROWS, K, false);
+		p.gemv_row_parts = 1;
 		return p;
 	}
 	if (gemv_rows_suits(M, N, K)) {

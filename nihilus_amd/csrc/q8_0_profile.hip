@@ -7,7 +7,7 @@
 // Batch runner: a list of mul_mat operations enqueued from native code in one call, so a decode step's
 // launches (7 projections x 32 layers + lm_head at LLaMA-3-8B) are not paced by the caller's language runtime.
 #include "../../include/nihilus_amd/q8_0_abi.h"
-#include "q8_0_device.h"
+#include "q8_0_plan.h"
 
 #include <atomic>
 #include <mutex>
@@ -265,8 +265,8 @@ int nh_q8_0_mul_mat_batch(const nh_q8_0_mul_mat_op* host_ops, int64_t count, voi
 			i += g;
 			continue;
 		}
-		if (nh::gemv_rows_suits(op.M, op.N, op.K)) {
-			// a few rows: still the mat-vec kernel (one dot product per row), quantize inside, the workspace stays unused
+		if (!nh::plan_mul_mat(op.M, op.N, op.K).quantize_launch) {
+			// a few rows: still a mat-vec kernel (quantize inside), the workspace stays unused
 			const int rc = nh_q8_0_mul_mat(op.W_tiled, op.x, op.y, op.M, op.N, op.K, workspace, workspace_bytes, stream);
 			if (rc != NH_OK) {
 				return rc;

@@ -38,7 +38,7 @@ def tiled_bytes(rows: int, k: int) -> int:
     return n
 
 
-KERNEL_NAMES = {0: "nothing", 1: "gemv", 2: "gemv_rows", 3: "gemm_skinny", 4: "gemm_tile_stream", 5: "gemm_tile"}
+KERNEL_NAMES = {0: "nothing", 1: "gemv", 2: "gemv_rows", 3: "gemm_skinny", 4: "gemm_tile_stream", 5: "gemm_tile", 6: "gemv_rows_mfma"}
 
 
 def plan_mul_mat(m: int, n: int, k: int) -> dict:
@@ -48,7 +48,7 @@ def plan_mul_mat(m: int, n: int, k: int) -> dict:
     raw = (ctypes.c_int32 * 8)()
     _lib.check("nh_q8_0_debug_plan_mul_mat", _lib.lib().nh_q8_0_debug_plan_mul_mat(m, n, k, raw))
     plan = {"kernel": KERNEL_NAMES[raw[0]], "quantize_launch": bool(raw[1])}
-    if raw[0] == 1:
+    if raw[0] in (1, 6):
         plan.update(k_splits=raw[2], groups_per_wave=raw[3], row_parts=raw[4])
     elif raw[0] == 3:
         plan.update(activation_strips=raw[2], k_splits=raw[3])

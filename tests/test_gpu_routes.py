@@ -18,15 +18,17 @@ ROUTES = [
     (1, 4096, 4096, "gemv", {"k_splits": 1, "row_parts": 2}),
     (1, 14336, 4096, "gemv", {"k_splits": 1, "row_parts": 1}),
     (3, 14336, 4096, "gemv_rows", {}),
-    (5, 1024, 8192, "gemv_rows", {}),  # the wide form on a small matrix
-    (8, 4096, 4096, "gemm_skinny", {"activation_strips": 1, "k_splits": 1}),
+    (5, 1024, 8192, "gemv_rows_mfma", {"k_splits": 4}),  # the rows as an MFMA operand, quantize inside; few strips: K over four workgroups
+    (8, 4096, 4096, "gemv_rows_mfma", {"k_splits": 2, "groups_per_wave": 1}),
+    (4, 14336, 4096, "gemv_rows_mfma", {"k_splits": 1, "groups_per_wave": 2}),
+    (8, 14336, 4096, "gemm_skinny", {"activation_strips": 1, "k_splits": 1}),
     (32, 4096, 14336, "gemm_skinny", {"activation_strips": 1, "k_splits": 2}),  # K over two workgroups per strip, arrival counter
     (128, 4096, 4096, "gemm_skinny", {"activation_strips": 2, "k_splits": 1}),  # more than 64 rows walked in groups of 64
     (64, 20480, 4096, "gemm_skinny", {"activation_strips": 2}),  # 160 column blocks whose K the tile kernel could not split
     (64, 14336, 4096, "gemm_tile_stream", {"activation_strips": 2, "k_sets": 4, "k_splits": 2}),
     (16, 8192, 8192, "gemm_tile_stream", {"activation_strips": 1, "k_sets": 4, "k_splits": 4}),
     (64, 4096, 14336, "gemm_tile_stream", {"activation_strips": 2, "k_sets": 4, "k_splits": 4}),
-    (8, 24576, 1024, "gemm_tile_stream", {"activation_strips": 1, "k_splits": 1}),  # 192 column blocks: the tile kernel at any M
+    (16, 24576, 1024, "gemm_tile_stream", {"activation_strips": 1, "k_splits": 1}),  # 192 column blocks: the tile kernel from nine rows on
     (512, 4096, 4096, "gemm_tile", {"activation_strips": 2, "k_sets": 4}),
     (128, 20480, 4096, "gemm_tile", {"activation_strips": 2, "k_sets": 2}),
     (512, 14336, 4096, "gemm_tile", {"activation_strips": 2, "k_sets": 1}),

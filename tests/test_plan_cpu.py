@@ -33,17 +33,27 @@ def test_mat_vec_cut_of_the_decode_shapes():
         assert (p["k_splits"], p["groups_per_wave"], p["row_parts"]) == (splits, tiles, parts), (n, k, p)
 
 
-def test_small_batches_on_small_matrices_stay_on_the_mat_vec_kernel():
-    # up to 5 rows on matrices of at most 40 MB: the quantize launch in front of the MFMA kernel would cost more than the dots
+def test_four_to_eight_rows_on_small_matrices_take_the_mfma_mat_vec():
+    # no quantize launch, no workspace: up to 8 rows on matrices of at most 40 MB, 4 rows up to 80 MB; beyond that the quantize launch
+    # and the MFMA kernels (every strip's workgroup quantizing the rows again would cost more than the launch)
     for n, k in (L8B["q_o"], L8B["k_v"], L70B["k_v"]):
-        assert kernel(4, n, k) == "gemv_rows" and kernel(5, n, k) == "gemv_rows" and kernel(6, n, k) == "gemm_skinny"
-    for n, k in (L8B["gate_up"], L8B["down"], L70B["q_o"], L70B["gate_up"]):
-        assert kernel(4, n, k) != "gemv_rows"
+        for m in (4, 5, 8):
+            p = q8_0.plan_mul_mat(m, n, k)
+            assert p["kernel"] == "gemv_rows_mfma" and not p["quantize_launch"], (m, n, k)
+        assert kernel(9, n, k) == "gemm_skinny"
+    for n, k in (L8B["gate_up"], L8B["down"], L70B["q_o"]):
+        assert kernel(4, n, k) == "gemv_rows_mfma" and kernel(5, n, k) != "gemv_rows_mfma" and kernel(8, n, k) != "gemv_rows_mfma"
+    for n, k in (L70B["gate_up"], L70B["down"], L70B["lm_head"], L8B["lm_head"]):
+        assert kernel(4, n, k) not in ("gemv_rows", "gemv_rows_mfma")
+    # its cut: a workgroup per CU where K allows it, a wave at most two groups
+    assert q8_0.plan_mul_mat(8, 4096, 4096)["k_splits"] == 2 and q8_0.plan_mul_mat(8, 4096, 4096)["groups_per_wave"] == 1
+    assert q8_0.plan_mul_mat(4, 1024, 8192)["k_splits"] == 4
+    assert q8_0.plan_mul_mat(4, 14336, 4096)["k_splits"] == 1 and q8_0.plan_mul_mat(4, 14336, 4096)["groups_per_wave"] == 2
 
 
 def test_crossover_shapes():
     # BASELINE configs[2]: M in {1, 8, 32, 128, 512} on [4096 x 4096] and [14336 x 4096]
-    assert [kernel(m, 4096, 4096) for m in (1, 8, 32, 128, 512)] == ["gemv", "gemm_skinny", "gemm_skinny", "gemm_skinny", "gemm_tile"]
+    assert [kernel(m, 4096, 4096) for m in (1, 8, 32, 128, 512)] == ["gemv", "gemv_rows_mfma", "gemm_skinny", "gemm_skinny", "gemm_tile"]
     assert [kernel(m, 14336, 4096) for m in (1, 8, 32, 128, 512)] == ["gemv", "gemm_skinny", "gemm_skinny", "gemm_tile", "gemm_tile"]
     p = q8_0.plan_mul_mat(512, 4096, 4096)  # a grid short of four waves per SIMD: four K sets per workgroup
     assert (p["activation_strips"], p["k_sets"], p["k_splits"], p["grid"]) == (2, 4, 1, (32, 8))
@@ -54,8 +64,8 @@ def test_crossover_shapes():
 def test_batched_decode_at_the_70b_shapes():
     # BASELINE configs[4]: M in {4, 16, 64}
     want = {
-        "q_o": ["gemm_skinny", "gemm_tile_stream", "gemm_tile_stream"],
-        "k_v": ["gemv_rows", "gemm_skinny", "gemm_skinny"],
+        "q_o": ["gemv_rows_mfma", "gemm_tile_stream", "gemm_tile_stream"],
+        "k_v": ["gemv_rows_mfma", "gemm_skinny", "gemm_skinny"],
         "gate_up": ["gemm_tile_stream"] * 3,
         "down": ["gemm_skinny", "gemm_tile_stream", "gemm_tile_stream"],
         "lm_head": ["gemm_tile_stream"] * 3,
