@@ -59,15 +59,50 @@ __device__ __forceinline__ int quantize_value(float f, float id) {
 	return max(-128, min(127, q));
 }
 
-// One lane's share of quantize_row_q8_0 (reference cpu/avx_2.hpp:4439-4489): eight consecutive lanes hold one
-// 32-value block as eight float4.  Returns this lane's four quants packed little-endian; *dh = fp16 bits of d.
+// A value from another lane of the same row of 16 lanes, by a fixed pattern (data-parallel primitive: no LDS traffic, and it
+// folds into the instruction that uses it).  All lanes involved must be active.
+template<int CTRL> __device__ __forceinline__ float lane_pattern(float x) {
+	return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+constexpr int DPP_QUAD_SWAP_1	 = 0xB1; // quad_perm [1, 0, 3, 2]: lane ^ 1
+constexpr int DPP_QUAD_SWAP_2	 = 0x4E; // quad_perm [2, 3, 0, 1]: lane ^ 2
+constexpr int DPP_ROW_HALF_MIRROR = 0x141; // lane i <-> 7 - i within each group of eight: pairs the two quads of the group
+
+// One lane's share of quantize_row_q8_0 (reference cpu/avx_2.hpp:4439-4489): eight consecutive lanes (a group aligned to eight)
+// hold one 32-value block as eight float4.  Returns this lane's four quants packed little-endian; *dh = fp16 bits of d.
 //   amax = max|x_i|; d = fp16_rne(amax / 127.f); id = amax != 0 ? 127.f / amax : 0; q_i = int8(rne(fl32(x_i * id)))
 // Divide, multiply and rounding are separate correctly rounded fp32 operations; all eight lanes must be active.
+// Two routes to the same bits.  The general one spells the operations out with every guard the corner cases need (NaN and
+// infinity among the values, 127 / amax overflowing, quotients near the subnormal range).  The short one runs when no lane of the
+// wave has such a block -- every value finite, amax zero or within [2^-60, 2^60]:
+//   * amax / 127 as q = amax * c, r = fma(-127, q, amax), d = fma(r, c, q) with c = fl32(1 / 127): with the correctly rounded
+//     reciprocal of the divisor and the exact remainder from the fma, one correction step gives the correctly rounded quotient;
+//   * 127 / amax as the reciprocal estimate, one refinement of it and two of the quotient -- the steps of the general
+//     division, without its rescaling and special-case handling, which are the identity in this range;
+//   * |x_i * id| <= 127 (1 + 2^-23), so the rounded product converts to int8 without the NaN guard and the clamp.
 __device__ __forceinline__ uint32_t quantize_block_lane(float4 v, uint16_t* dh) {
 	float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-	amax	   = fmaxf(amax, __shfl_xor(amax, 1));
-	amax	   = fmaxf(amax, __shfl_xor(amax, 2));
-	amax	   = fmaxf(amax, __shfl_xor(amax, 4));
+	amax	   = fmaxf(amax, lane_pattern<DPP_QUAD_SWAP_1>(amax));
+	amax	   = fmaxf(amax, lane_pattern<DPP_QUAD_SWAP_2>(amax));
+	amax	   = fmaxf(amax, lane_pattern<DPP_ROW_HALF_MIRROR>(amax));
+	const float sum = (v.x + v.y) + (v.z + v.w); // NaN or infinity among the four makes this NaN or infinite
+	const bool plain = (amax == 0.0f || (amax >= 0x1p-60f && amax <= 0x1p60f)) && fabsf(sum) <= 0x1p100f;
+	if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
+		constexpr float c = 1.0f / 127.0f; // correctly rounded by the compiler
+		const float q	  = __fmul_rn(amax, c);
+		const float d	  = fmaf(fmaf(-127.0f, q, amax), c, q);
+		const float y0	  = __builtin_amdgcn_rcpf(amax);
+		const float y1	  = fmaf(fmaf(-amax, y0, 1.0f), y0, y0);
+		const float q0	  = __fmul_rn(127.0f, y1);
+		const float q1	  = fmaf(fmaf(-amax, q0, 127.0f), y1, q0);
+		const float q2	  = fmaf(fmaf(-amax, q1, 127.0f), y1, q1);
+		const float id	  = amax != 0.0f ? q2 : 0.0f;
+		*dh				  = float_to_half_bits(d);
+		const uint32_t a = static_cast<uint32_t>(static_cast<int>(rintf(__fmul_rn(v.x, id)))), b = static_cast<uint32_t>(static_cast<int>(rintf(__fmul_rn(v.y, id))));
+		const uint32_t e = static_cast<uint32_t>(static_cast<int>(rintf(__fmul_rn(v.z, id)))), f = static_cast<uint32_t>(static_cast<int>(rintf(__fmul_rn(v.w, id))));
+		// low bytes of a, b into bytes 0, 1; of e, f into bytes 2, 3 (selector: 0..3 = bytes of the second operand, 4..7 of the first, 0x0c = zero)
+		return __builtin_amdgcn_perm(b, a, 0x0c0c0400u) | __builtin_amdgcn_perm(f, e, 0x04000c0cu);
+	}
 	const float d  = __fdiv_rn(amax, 127.0f);
 	const float id = (amax != 0.0f) ? __fdiv_rn(127.0f, amax) : 0.0f;
 	*dh			   = float_to_half_bits(d);
