@@ -198,3 +198,17 @@ def test_generator_statistics_and_determinism(oracle):
     assert np.array_equal(w, oracle.fill_weights(0, 64, 4096))
     assert np.array_equal(oracle.fill_weights(0, 32, 4096, first_block=32 * 128), w[32 * 128 * 34 :])
     assert not np.array_equal(w, oracle.fill_weights(1, 64, 4096))
+
+
+def test_division_by_127_through_the_rounded_reciprocal_is_exact(tmp_path):
+    """The device quantizer's short route: amax / 127 as reciprocal multiply + one fma correction.  Checked on the host against the
+    correctly rounded division for every fp32 mantissa (tests/cpp/divide_by_127_check.c)."""
+    import os
+    import subprocess
+
+    src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "divide_by_127_check.c")
+    exe = str(tmp_path / "divide_by_127_check")
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-mfma", "-o", exe, src, "-lm"], check=True)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout
+    assert "mismatches 0" in res.stdout
