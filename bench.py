@@ -569,7 +569,7 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
         shapes = [(4096, K), (14336, K)]
         ws = [q8_0.tile(q8_0.fill_weight_blocks(3 + i, n, k), n, k) for i, (n, k) in enumerate(shapes)]
         rows = []
-        for m in (1, 2, 4, 8, 32, 64, 128, 512):
+        for m in (1, 2, 4, 8, 16, 32, 64, 128, 512):
             xm = x[:m].contiguous()
             ws_bytes = max(256, lib.nh_q8_0_mul_mat_workspace_bytes(m, K))
             wsp = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)

@@ -264,7 +264,7 @@ int nh_q8_0_gemm_tiled_gate_up_silu(const void* W_gate_tiled, const void* W_up_t
 /* Scratch the fused call needs for the quantized activations (device bytes, 256-byte aligned by the caller);
  * 0 for M <= 3, where the quantize happens inside the mat-vec kernel and workspace may be NULL. */
 int64_t nh_q8_0_mul_mat_workspace_bytes(int64_t M, int64_t K);
-/* quantize(x) then GEMV (M == 1; M = 2, 3: the same kernel with one dot product per row; M = 4 ... 8 on matrices up to 40 MB, M = 4 up to
+/* quantize(x) then GEMV (M == 1; M = 2, 3: the same kernel with one dot product per row; M = 4 ... 16 on matrices up to 40 MB, M = 4 up to
  * 80 MB: the same kernel with the rows as an MFMA operand -- all of these quantize inside the kernel and leave the workspace
  * untouched) or GEMM (otherwise: a quantize launch into the workspace, then an MFMA kernel) against a tiled weight: the whole
  * rms_norm-output -> projection step of core_traits.hpp:575-594 / :976-989 as one call. */
@@ -342,7 +342,7 @@ int nh_q8_0_debug_ffn_gate_up(float* gate_out, float* up_out, int64_t N_ff, void
  * Needs no GPU.  host_plan receives eight int32:
  *   [0] kernel: 0 nothing (empty problem), 1 fused quantize + streaming mat-vec (M == 1), 2 the same kernel with one dot product
  *       per row (a few rows), 3 weight-streaming MFMA kernel, 4 MFMA tile kernel with non-temporal weights (batched decode on
- *       large matrices), 5 MFMA tile kernel (prefill), 6 the streaming mat-vec with four to eight rows as an MFMA operand, quantize
+ *       large matrices), 5 MFMA tile kernel (prefill), 6 the streaming mat-vec with four to sixteen rows as an MFMA operand, quantize
  *       inside (small matrices);
  *   [1] 1 when the activations are quantized by a launch of their own into the workspace (kernels 3, 4, 5);
  *   kernel 1, 6: [2] workgroups per 32-row strip along K, [3] 128-quant groups per wave, [4] row parts per strip;

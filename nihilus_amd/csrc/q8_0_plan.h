@@ -17,7 +17,7 @@ enum mul_mat_kernel : int {
 	MM_GEMM_SKINNY		= 3, // quantize launch + weight-streaming MFMA kernel (gemm_skinny_kernel)
 	MM_GEMM_TILE_STREAM = 4, // quantize launch + MFMA tile kernel with non-temporal weight loads (batched decode on large matrices)
 	MM_GEMM_TILE		= 5, // quantize launch + MFMA tile kernel (prefill)
-	MM_GEMV_ROWS_MFMA	= 6, // 4..8 rows on small matrices: the streaming mat-vec with the rows as an MFMA operand (gemv_rows8_kernel), quantize inside
+	MM_GEMV_ROWS_MFMA	= 6, // 4..16 rows on small matrices: the streaming mat-vec with the rows as an MFMA operand (gemv_rows8_kernel), quantize inside
 };
 
 constexpr int SK_WAVES			  = 8; // waves per workgroup of the weight-streaming MFMA kernel
@@ -158,31 +158,32 @@ inline bool plan_gate_up_fused(int64_t M, int64_t n_ff, int64_t K, gemm_tile_cut
 	return true;
 }
 
-// The eight-row MFMA mat-vec's cut (q8_0_gemv_rows_mfma.hip): K over workgroups until a wave owns at most two groups (its
-// register budget), within the split scratch's units (one per strip, activation row and split); matrices with few strips are cut
+// The MFMA mat-vec's cut (q8_0_gemv_rows_mfma.hip): K over workgroups until a wave owns at most two groups (one with the
+// sixteen-row operand: its register budget), within the split scratch's units (one per strip, activation row and split); matrices with few strips are cut
 // further so that the launch reaches the CUs.  Under HIP graph capture: no K split (a replay could not renew the hand-off's epoch),
 // a chunked walk instead.
-constexpr int GEMV_ROWS_MFMA_MAX = 8;
-// Where it is the fastest form (measured against what ran before, quantize launch included; us):
-//   [4096 x 4096]   17.8 MB   M = 4:  6.0 against  8.1 (dot-product kernel)      M = 8:  7.5 against 12.2 (quantize + streaming MFMA kernel)
-//   [1024 x 8192]    8.9 MB   M = 4:  6.0 against  7.3
-//   [14336 x 4096]  62.4 MB   M = 4: 14.5 against 15.6                            M = 8: 19.3 against 15.7
-//   [8192 x 8192]   71.3 MB   M = 4: 18.4 against 21.2
-//   [28672 x 8192]   250 MB   M = 4: 51   against 43.6;  [128256 x 8192]: 199 against 167
-// Every strip's workgroup quantizes all the rows again, which costs in proportion to M and to the matrix: up to eight rows on
+constexpr int GEMV_ROWS_MFMA_MAX = 16;
+// Where it is the fastest form (measured against what ran before, quantize launch included; us, new / old):
+//   [4096 x 4096]   17.8 MB   M = 4:  5.2 /  8.1 (dot-product kernel)   M = 8:  6.8 / 12.2   M = 16:  8.6 / 11.7 (quantize + streaming MFMA kernel)
+//   [1024 x 8192]    8.9 MB   M = 4:  5.6 /  7.3                        M = 16:  9.1 / 14.3
+//   [14336 x 4096]  62.4 MB   M = 4: 13.7 / 15.6                        M = 8:  19.3 / 15.7
+//   [8192 x 8192]   71.3 MB   M = 4: 17.4 / 21.2
+//   [28672 x 8192]   250 MB   M = 4: 51   / 43.6;  [128256 x 8192]: 199 / 167
+// Every strip's workgroup quantizes all the rows again, which costs in proportion to M and to the matrix: up to sixteen rows on
 // matrices of at most 40 MB, four on matrices of at most 80 MB.  (Two and three rows stay on the dot-product kernel.)
 inline bool gemv_rows_mfma_suits(int64_t M, int64_t N, int64_t K) {
 	const int64_t weight_bytes = N * (K / QK) * BLOCK_BYTES;
 	return M >= 4 && M <= GEMV_ROWS_MFMA_MAX && (weight_bytes <= (int64_t{ 40 } << 20) || (M == 4 && weight_bytes <= (int64_t{ 80 } << 20)));
 }
-inline gemv_plan plan_gemv_rows_mfma(int64_t strips, int64_t K, bool capturing) {
+inline gemv_plan plan_gemv_rows_mfma(int64_t strips, int64_t K, int rows, bool capturing) { // rows: 8 or 16, the kernel's operand rows
 	gemv_plan p;
 	p.strips	   = static_cast<int>(strips);
 	p.groups	   = static_cast<int>(K / GROUP_K);
 	p.splits	   = 1;
 	auto tiles_for = [&](int sp) { return (p.groups + GEMV_WAVES * sp - 1) / (GEMV_WAVES * sp); };
-	auto room	   = [&](int sp) { return strips * GEMV_ROWS_MFMA_MAX * sp <= GEMV_MAX_SPLIT_UNITS; };
-	while (tiles_for(p.splits) > 2 && room(p.splits * 2)) {
+	auto room	   = [&](int sp) { return strips * rows * sp <= GEMV_MAX_SPLIT_UNITS; };
+	const int fit  = rows <= 8 ? 2 : 1; // groups of a wave's K range that its registers hold at once
+	while (tiles_for(p.splits) > fit && room(p.splits * 2)) {
 		p.splits *= 2;
 	}
 	// (a workgroup per CU, not per two as in the dot-product kernel: every workgroup quantizes its K range of all the rows, and that
@@ -228,7 +229,7 @@ inline mul_mat_plan plan_mul_mat(int64_t M, int64_t N, int64_t K) {
 	}
 	if (gemv_rows_mfma_suits(M, N, K)) {
 		p.kernel		 = MM_GEMV_ROWS_MFMA;
-		p.gemv			 = plan_gemv_rows_mfma((N + STRIP_ROWS - 1) / STRIP_ROWS, K, false);
+		p.gemv			 = plan_gemv_rows_mfma((N + STRIP_ROWS - 1) / STRIP_ROWS, K, M <= 8 ? 8 : 16, false);
 		p.gemv_row_parts = 1;
 		return p;
 	}

@@ -1,4 +1,4 @@
-"""GPU: four to eight activation rows on small matrices -- the streaming mat-vec with the rows as an MFMA operand, the activation
+"""GPU: four to sixteen activation rows on small matrices -- the streaming mat-vec with the rows as an MFMA operand, the activation
 quantize inside the kernel (q8_0_gemv_rows_mfma.hip), reached through nh_q8_0_mul_mat.
 
 Checked against the CPU checker's quantize + mat-mat (1e-4 relative L2 overall and row by row), for every row count the kernel
@@ -28,7 +28,7 @@ def test_rows_on_the_matrix_cores_match_the_checker(q8, oracle, n, k):
     rng = np.random.default_rng(n + k)
     w = random_blocks(rng, n, k, 0.02)
     wt = q8.tile(to_dev(w), n, k)
-    for m in ((4, 5, 6, 7, 8) if n * (k // 32) * 34 <= 40 << 20 else (4,)):  # above 40 MB the kernel takes four rows only
+    for m in ((4, 5, 6, 7, 8, 9, 11, 16) if n * (k // 32) * 34 <= 40 << 20 else (4,)):  # above 40 MB the kernel takes four rows only
         assert q8.plan_mul_mat(m, n, k)["kernel"] == "gemv_rows_mfma"
         x = rng.standard_normal((m, k)).astype(np.float32)
         x[m - 1, : k // 2] *= 37.0  # rows of different magnitude: every row has its own block scales
@@ -53,20 +53,22 @@ def test_rows_of_zeros_and_an_absent_scale(q8, oracle):
     rng = np.random.default_rng(5)
     w = random_blocks(rng, n, k, 0.02)
     wt = q8.tile(to_dev(w), n, k)
-    x = rng.standard_normal((6, k)).astype(np.float32)
+    x = rng.standard_normal((11, k)).astype(np.float32)
+    x[9] = 0.0
     x[2] = 0.0  # amax = 0: scale 0, quants 0 (the reference's guard against 127 / 0)
     x[4, 32:64] = 0.0  # one block of zeros inside a row
     y = to_host(q8.mul_mat(wt, to_dev(x), n, k))
-    assert np.array_equal(y[2], np.zeros(n, dtype=np.float32))
+    assert np.array_equal(y[2], np.zeros(n, dtype=np.float32)) and np.array_equal(y[9], np.zeros(n, dtype=np.float32))
     assert rel_l2(y, _want(oracle, w, x, n, k)) <= REL_L2_TOL
 
 
-def test_captured_stream_takes_the_unsplit_walk(q8, oracle):
+@pytest.mark.parametrize("m", [8, 16])
+def test_captured_stream_takes_the_unsplit_walk(q8, oracle, m):
     # under capture the K split's hand-off (an epoch per launch) cannot be used: the same kernel walks K in chunks instead
     from nihilus_amd import _lib
 
     _lib.check("nh_q8_0_prepare", _lib.lib().nh_q8_0_prepare())
-    n, k, m = 1024, 8192, 8
+    n, k = 1024, 8192
     assert q8.plan_mul_mat(m, n, k)["k_splits"] == 4
     rng = np.random.default_rng(9)
     w = random_blocks(rng, n, k, 0.02)

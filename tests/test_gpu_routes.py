@@ -20,6 +20,8 @@ ROUTES = [
     (3, 14336, 4096, "gemv_rows", {}),
     (5, 1024, 8192, "gemv_rows_mfma", {"k_splits": 4}),  # the rows as an MFMA operand, quantize inside; few strips: K over four workgroups
     (8, 4096, 4096, "gemv_rows_mfma", {"k_splits": 2, "groups_per_wave": 1}),
+    (16, 4096, 4096, "gemv_rows_mfma", {"k_splits": 2, "groups_per_wave": 1}),  # the sixteen-row form of the operand tile
+    (13, 1024, 14336, "gemv_rows_mfma", {"k_splits": 8, "groups_per_wave": 1}),
     (4, 14336, 4096, "gemv_rows_mfma", {"k_splits": 1, "groups_per_wave": 2}),
     (8, 14336, 4096, "gemm_skinny", {"activation_strips": 1, "k_splits": 1}),
     (32, 4096, 14336, "gemm_skinny", {"activation_strips": 1, "k_splits": 2}),  # K over two workgroups per strip, arrival counter
@@ -28,7 +30,7 @@ ROUTES = [
     (64, 14336, 4096, "gemm_tile_stream", {"activation_strips": 2, "k_sets": 4, "k_splits": 2}),
     (16, 8192, 8192, "gemm_tile_stream", {"activation_strips": 1, "k_sets": 4, "k_splits": 4}),
     (64, 4096, 14336, "gemm_tile_stream", {"activation_strips": 2, "k_sets": 4, "k_splits": 4}),
-    (16, 24576, 1024, "gemm_tile_stream", {"activation_strips": 1, "k_splits": 1}),  # 192 column blocks: the tile kernel from nine rows on
+    (24, 24576, 1024, "gemm_tile_stream", {"activation_strips": 1, "k_splits": 1}),  # 192 column blocks: the tile kernel from seventeen rows on
     (512, 4096, 4096, "gemm_tile", {"activation_strips": 2, "k_sets": 4}),
     (128, 20480, 4096, "gemm_tile", {"activation_strips": 2, "k_sets": 2}),
     (512, 14336, 4096, "gemm_tile", {"activation_strips": 2, "k_sets": 1}),

@@ -33,14 +33,14 @@ def test_mat_vec_cut_of_the_decode_shapes():
         assert (p["k_splits"], p["groups_per_wave"], p["row_parts"]) == (splits, tiles, parts), (n, k, p)
 
 
-def test_four_to_eight_rows_on_small_matrices_take_the_mfma_mat_vec():
-    # no quantize launch, no workspace: up to 8 rows on matrices of at most 40 MB, 4 rows up to 80 MB; beyond that the quantize launch
+def test_four_to_sixteen_rows_on_small_matrices_take_the_mfma_mat_vec():
+    # no quantize launch, no workspace: up to 16 rows on matrices of at most 40 MB, 4 rows up to 80 MB; beyond that the quantize launch
     # and the MFMA kernels (every strip's workgroup quantizing the rows again would cost more than the launch)
     for n, k in (L8B["q_o"], L8B["k_v"], L70B["k_v"]):
-        for m in (4, 5, 8):
+        for m in (4, 5, 8, 9, 16):
             p = q8_0.plan_mul_mat(m, n, k)
             assert p["kernel"] == "gemv_rows_mfma" and not p["quantize_launch"], (m, n, k)
-        assert kernel(9, n, k) == "gemm_skinny"
+        assert kernel(17, n, k) == "gemm_skinny"
     for n, k in (L8B["gate_up"], L8B["down"], L70B["q_o"]):
         assert kernel(4, n, k) == "gemv_rows_mfma" and kernel(5, n, k) != "gemv_rows_mfma" and kernel(8, n, k) != "gemv_rows_mfma"
     for n, k in (L70B["gate_up"], L70B["down"], L70B["lm_head"], L8B["lm_head"]):
@@ -49,6 +49,9 @@ def test_four_to_eight_rows_on_small_matrices_take_the_mfma_mat_vec():
     assert q8_0.plan_mul_mat(8, 4096, 4096)["k_splits"] == 2 and q8_0.plan_mul_mat(8, 4096, 4096)["groups_per_wave"] == 1
     assert q8_0.plan_mul_mat(4, 1024, 8192)["k_splits"] == 4
     assert q8_0.plan_mul_mat(4, 14336, 4096)["k_splits"] == 1 and q8_0.plan_mul_mat(4, 14336, 4096)["groups_per_wave"] == 2
+    # nine to sixteen rows: one group per wave at a time (the rows' fp32 slices share the registers with the weight tiles)
+    assert q8_0.plan_mul_mat(16, 4096, 4096)["k_splits"] == 2 and q8_0.plan_mul_mat(16, 4096, 4096)["groups_per_wave"] == 1
+    assert q8_0.plan_mul_mat(16, 1024, 8192)["k_splits"] == 4
 
 
 def test_crossover_shapes():
@@ -65,7 +68,7 @@ def test_batched_decode_at_the_70b_shapes():
     # BASELINE configs[4]: M in {4, 16, 64}
     want = {
         "q_o": ["gemv_rows_mfma", "gemm_tile_stream", "gemm_tile_stream"],
-        "k_v": ["gemv_rows_mfma", "gemm_skinny", "gemm_skinny"],
+        "k_v": ["gemv_rows_mfma", "gemv_rows_mfma", "gemm_skinny"],
         "gate_up": ["gemm_tile_stream"] * 3,
         "down": ["gemm_skinny", "gemm_tile_stream", "gemm_tile_stream"],
         "lm_head": ["gemm_tile_stream"] * 3,
