@@ -72,9 +72,10 @@ inline gemm_skinny_cut plan_gemm_skinny(int64_t M, int64_t N, int64_t K) {
 	c.splits			= 1;
 	// The hand-off between workgroups is expensive here (a partial tile of 16 values per lane and strip, an arrival counter,
 	// the last arriver reading every share): K goes over several workgroups only until every CU has one (and every wave
-	// keeps at least four groups), or when a wave would otherwise walk more than sixteen groups.  Measured on [8192 x 28672]
-	// at M = 16: 68 us with eight workgroups per strip, 51 us with two.
-	while (units * c.splits < 256 && groups >= 8 * SK_WAVES * c.splits && units * c.splits * 2 <= SK_MAX_SPLIT_UNITS && units <= SK_MAX_SPLIT_STRIPS) {
+	// keeps at least two groups, one step of the kernel's walk: [4096 x 4096] at M = 32 12.1 -> 10.8 us, [1024 x 8192] at M = 64
+	// 14.9 -> 13.2 us against keeping four), or when a wave would otherwise walk more than sixteen groups.  Measured on
+	// [8192 x 28672] at M = 16: 68 us with eight workgroups per strip, 51 us with two.
+	while (units * c.splits < 256 && groups >= 4 * SK_WAVES * c.splits && units * c.splits * 2 <= SK_MAX_SPLIT_UNITS && units <= SK_MAX_SPLIT_STRIPS) {
 		c.splits *= 2;
 	}
 	while (groups > 16 * SK_WAVES * c.splits && units * c.splits * 2 <= SK_MAX_SPLIT_UNITS && units <= SK_MAX_SPLIT_STRIPS) {
