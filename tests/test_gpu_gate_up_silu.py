@@ -77,4 +77,9 @@ def test_gate_up_silu_arguments(q8):
     assert lib.nh_q8_0_gemm_tiled_gate_up_silu(w.data_ptr(), w.data_ptr(), a.data_ptr(), out.data_ptr(), None, 0, 37, 3584, 1024, None) == -6
     assert lib.nh_q8_0_gemm_tiled_gate_up_silu(w.data_ptr(), w.data_ptr(), a.data_ptr(), None, None, 0, 37, 3584, 1024, None) == -1
     assert lib.nh_q8_0_gemm_tiled_gate_up_silu(None, None, None, None, None, 0, 0, 3584, 1024, None) == 0
+    # an empty inner dimension: gate = up = 0, silu(0) * 0 = 0, every block of the output is a zero block (scale 0, quants 0)
+    ws = torch.empty(lib.nh_q8_0_gate_up_silu_workspace_bytes(37, 3584, 0), dtype=torch.uint8, device="cuda")
+    out.fill_(0xFF)
+    assert lib.nh_q8_0_gemm_tiled_gate_up_silu(None, None, None, out.data_ptr(), ws.data_ptr(), ws.numel(), 37, 3584, 0, None) == 0
     torch.cuda.synchronize()
+    assert not out.cpu().numpy().any()
