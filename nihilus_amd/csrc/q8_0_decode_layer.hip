@@ -159,12 +159,13 @@ __device__ __forceinline__ void store_row(float* __restrict__ y, uint64_t* __res
 	__hip_atomic_store(&y_tagged[row], (static_cast<uint64_t>(epoch) << 32) | __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// PAIR: every gate/up wave takes both matrices.
-template<bool PAIR> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_layer_kernel(layer_args a) {
+// Every gate/up wave takes a K range of both matrices (one staged slice of the input row for the two), two groups of each at a time:
+// CHUNKS = 1 for hidden states up to 4096 values (a wave's whole share in one go), 2 up to 8192.
+template<int CHUNKS> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_layer_kernel(layer_args a) {
 	__shared__ __align__(16) uint8_t xs_q[GEMV_WAVES][CHAIN_DOWN_ROWS_TILES * GROUP_K];
 	__shared__ float xs_d[GEMV_WAVES][CHAIN_DOWN_ROWS_TILES * GROUP_BLOCKS];
 	__shared__ float red[GEMV_WAVES][64];
-	__shared__ float red_up[PAIR ? GEMV_WAVES : 1][64];
+	__shared__ float red_up[GEMV_WAVES][64];
 	__shared__ float norm_red[16];
 	__shared__ __align__(16) float act_f[STRIP_ROWS];
 
@@ -172,7 +173,6 @@ template<bool PAIR> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_la
 	const int lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wg   = static_cast<int>(blockIdx.x);
-
 	if (wg < a.first_norm) {
 		// ---- attn_out: rows of W_o against Q(attn), + layer_in ----
 		const int strip = wg;
@@ -203,42 +203,34 @@ template<bool PAIR> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_la
 	if (wg < a.first_consumer) {
 		// ---- rows [32 * strip, + 32) of gate and of up against Q(n1) -> silu(g) * u -> activation block `strip` ----
 		const int strip		   = wg - a.first_producer;
-		const int matrix	   = PAIR ? 0 : wave >> 3;
-		const int slot		   = PAIR ? wave : wave & 7;
-		const int g0		   = slot * a.p_per_slot + min(slot, a.p_rem);
-		const int g1		   = g0 + a.p_per_slot + (slot < a.p_rem ? 1 : 0);
-		const uint8_t* w_strip = (matrix ? a.w_up : a.w_gate) + macro_offset(strip, 0, a.groups_e);
+		const int g0		   = wave * a.p_per_slot + min(wave, a.p_rem);
+		const int g1		   = g0 + a.p_per_slot + (wave < a.p_rem ? 1 : 0);
+		const uint8_t* w_strip = a.w_gate + macro_offset(strip, 0, a.groups_e);
+		const uint8_t* w_other = a.w_up + macro_offset(strip, 0, a.groups_e);
 		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
-		float acc = 0.0f;
-		[[maybe_unused]] float acc_up = 0.0f;
-		if constexpr (PAIR) {
+		float acc = 0.0f, acc_up = 0.0f;
+		if constexpr (CHUNKS == 1) {
 			acc = gemv_chunk<2, X_PUBLISHED_EARLY, DUMP_NONE, false, 1, 2>(w_strip, a.x_words, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_e, lane, row_l, a.n_ff, false, a.epoch, nullptr, 0,
-				a.spin_limit, a.w_up + macro_offset(strip, 0, a.groups_e), &acc_up);
-			red_up[wave][lane] = acc_up;
+				a.spin_limit, w_other, &acc_up);
 		} else {
-			for (int gc = g0; gc < g1; gc += CHAIN_TILES) {
-				acc += gemv_chunk<CHAIN_TILES, X_PUBLISHED_EARLY, DUMP_NONE, false>(w_strip, a.x_words, a.error_word, xs_q[wave], xs_d[wave], gc, min(CHAIN_TILES, g1 - gc), a.groups_e, lane, row_l, a.n_ff, false,
-					a.epoch, nullptr, 0, a.spin_limit);
-				__builtin_amdgcn_wave_barrier();
+			for (int gc = g0; gc < g1; gc += 2) {
+				float up_chunk = 0.0f;
+				acc += gemv_chunk<2, X_PUBLISHED_EARLY, DUMP_NONE, false, 1, 2>(w_strip, a.x_words, a.error_word, xs_q[wave], xs_d[wave], gc, min(2, g1 - gc), a.groups_e, lane, row_l, a.n_ff, false, a.epoch,
+					nullptr, 0, a.spin_limit, w_other, &up_chunk);
+				acc_up += up_chunk;
+				__builtin_amdgcn_wave_barrier(); // the next chunk overwrites this wave's LDS slices
 			}
 		}
+		red_up[wave][lane] = acc_up;
 		red[wave][lane] = acc;
 		__syncthreads();
 		if (wave == 0) {
 			if (lane < STRIP_ROWS) {
 				float g = 0.0f, u = 0.0f;
-				if constexpr (PAIR) {
 #pragma unroll
-					for (int w = 0; w < GEMV_WAVES; ++w) {
-						g += red[w][lane] + red[w][32 + lane];
-						u += red_up[w][lane] + red_up[w][32 + lane];
-					}
-				} else {
-#pragma unroll
-					for (int w = 0; w < GEMV_WAVES / 2; ++w) {
-						g += red[w][lane] + red[w][32 + lane];
-						u += red[GEMV_WAVES / 2 + w][lane] + red[GEMV_WAVES / 2 + w][32 + lane];
-					}
+				for (int w = 0; w < GEMV_WAVES; ++w) {
+					g += red[w][lane] + red[w][32 + lane];
+					u += red_up[w][lane] + red_up[w][32 + lane];
 				}
 				act_f[lane]									  = silu_mul(g, u);
 				a.gate_up[strip * STRIP_ROWS + lane]				  = g; // inspection copies, not read by this launch
@@ -457,11 +449,12 @@ hipError_t launch_decode_layer(const void* w_o, const float* attn, const float* 
 	// here the gate/up workgroups behind it fill the other CUs and have their weights on the way at once, and the CUs that start
 	// on attn_out run a few microseconds ahead of the rest from then on, so the chip's workgroups do not change rounds in lock-step
 	// (measured at the LLaMA-3-8B block: 43.1 us against 44.0 us with half strips).
-	// gate/up: sixteen K ranges per workgroup, both matrices per wave, where that is at most two groups a wave
-	const bool pair	  = (a.groups_e + GEMV_WAVES - 1) / GEMV_WAVES <= 2;
-	const int p_slots = pair ? GEMV_WAVES : GEMV_WAVES / 2;
-	a.p_per_slot	  = a.groups_e / p_slots;
-	a.p_rem			  = a.groups_e % p_slots;
+	// gate/up: sixteen K ranges per workgroup, both matrices per wave, two groups of each at a time: one such chunk covers a wave's
+	// share up to 4096 values of hidden state, two up to 8192 (CHAIN_MAX_EMBD).  (Up to 8192 the stage used to give eight waves to each
+	// matrix, four groups at a time: 128 registers and spills, the LLaMA-3-70B block 160.8 us against 150.3 us in this form.)
+	const bool one_chunk = (a.groups_e + GEMV_WAVES - 1) / GEMV_WAVES <= 2;
+	a.p_per_slot		 = a.groups_e / GEMV_WAVES;
+	a.p_rem				 = a.groups_e % GEMV_WAVES;
 	int splits = 1;
 	while ((a.groups_f + GEMV_WAVES * splits - 1) / (GEMV_WAVES * splits) > CHAIN_TILES) {
 		splits *= 2;
@@ -492,7 +485,7 @@ hipError_t launch_decode_layer(const void* w_o, const float* attn, const float* 
 	a.error_word	= sc.error_word;
 	a.spin_limit	= sc.spin_limit;
 	const dim3 block(GEMV_WAVES * 64);
-	return pair ? launch_kernel(KIND_GEMV, decode_layer_kernel<true>, dim3(grid), block, 0, s, a) : launch_kernel(KIND_GEMV, decode_layer_kernel<false>, dim3(grid), block, 0, s, a);
+	return one_chunk ? launch_kernel(KIND_GEMV, decode_layer_kernel<1>, dim3(grid), block, 0, s, a) : launch_kernel(KIND_GEMV, decode_layer_kernel<2>, dim3(grid), block, 0, s, a);
 }
 
 } // namespace nh

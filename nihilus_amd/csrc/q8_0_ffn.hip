@@ -301,7 +301,12 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 		return launch_ffn_t<4, false, true>(a, grid, s);
 	}
 	if (tiles > 4) {
-		return launch_ffn_t<4, true>(a, grid, s);
+		// the chunked walk in chunks of two groups: chunks of four leave the kernel at 128 registers with up to 14 spilled (the norm's
+		// registers on top of 72 for weights), and a spill's reload queues behind the weight loads like any other load.  Measured at
+		// the LLaMA-3-70B shapes: 133.0 -> 122.7 us with the norm in front, 116.3 -> 113.5 us without.  (Every wave taking both
+		// matrices, two groups of each at a time -- what the chained block's launch does with these shapes -- measured 124.2 and
+		// 117.1 us here: two spilled registers again.)
+		return launch_ffn_t<2, true>(a, grid, s);
 	}
 	if (tiles <= 1) {
 		return launch_ffn_t<1, false>(a, grid, s);

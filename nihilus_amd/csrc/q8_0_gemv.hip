@@ -501,6 +501,11 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 		}
 	}
 	if (p.tiles > 4) { // K too long to keep every load in flight within the scratch limits: chunked walk
+		if (x_is_f32 && norm_w) {
+			// chunks of two groups: with the norm's registers on top, chunks of four do not fit the 128 registers of a 1024-thread
+			// workgroup and the compiler spills, and a spill's reload queues behind the weight loads like any other load
+			return launch_gemv_tiled_t<2, true, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
+		}
 		return x_is_f32 ? launch_gemv_tiled_t<4, true, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s) : launch_gemv_tiled_t<4, false, true>(p, seg, x, dump, dump_mode, sc, norm_w, norm_eps, s);
 	}
 	const int tiles = p.tiles <= 1 ? 1 : (p.tiles <= 2 ? 2 : 4);

@@ -44,8 +44,8 @@ SHAPES = [
     (512, 1536, (512, 128, 128), False),  # a small block: few strips everywhere
     (1024, 3584, (4000,), False),  # last block -> logits, a ragged vocabulary
     (2048, 5632, (), False),  # nothing behind the block
-    (8192, 28672, (8192, 1024, 1024), True),  # LLaMA-3-70B block: whole attn_out strips in the separate launch too, so the same cuts everywhere
-    (8192, 3584, (1024, 256), False),  # the longest hidden state the one launch takes: four groups per wave, gate/up waves take one matrix each
+    (8192, 28672, (8192, 1024, 1024), False),  # LLaMA-3-70B block: a wave's three or four groups walked two at a time (another order of the sums than the separate launches')
+    (8192, 3584, (1024, 256), False),  # the longest hidden state the one launch takes: four groups per wave, gate/up in two chunks of two groups of both matrices
     (4096, 9216, (8000,), False),  # a row-cut down stage with a long, ragged stage behind it
     (4096, 14336, (1024,), False),  # ... and with a short one
 ]
