@@ -134,16 +134,18 @@ def test_few_rows_on_a_wide_matrix(q8, oracle, m, n, k):
 
 
 def test_mul_mat_batch_mixed_rows(q8, oracle):
-    # one native call, five projections: two mat-vecs sharing x (one launch), a 3-row op with no workspace use, two 8-row ops sharing the quantized x
+    # one native call, seven projections: two mat-vecs sharing x (one launch), a 3-row op and two 8-row ops with no workspace use (the
+    # quantize happens inside their kernels), two 24-row ops sharing the quantized x in the workspace
     import torch
 
     from nihilus_amd import _lib
 
-    k, shapes = 1024, [(1, 256), (1, 96), (3, 160), (8, 256), (8, 64)]
+    k, shapes = 1024, [(1, 256), (1, 96), (3, 160), (8, 256), (8, 64), (24, 256), (24, 64)]
     x1 = oracle.fill_activations(1, k).reshape(1, k)
     x3 = oracle.fill_activations(3, 3 * k).reshape(3, k)
     x8 = oracle.fill_activations(8, 8 * k).reshape(8, k)
-    xs = {1: x1, 3: x3, 8: x8}
+    x24 = oracle.fill_activations(24, 24 * k).reshape(24, k)
+    xs = {1: x1, 3: x3, 8: x8, 24: x24}
     xd = {m: to_dev(v) for m, v in xs.items()}
     ops = (_lib.MulMatOp * len(shapes))()
     keep, want = [], []
@@ -152,10 +154,11 @@ def test_mul_mat_batch_mixed_rows(q8, oracle):
         wt = q8.tile(to_dev(w), n, k)
         y = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
         keep += [wt, y]
-        ops[i] = _lib.MulMatOp(wt.data_ptr(), xd[m].data_ptr(), y.data_ptr(), m, n, k, 1 if i in (1, 4) else 0, 0)
+        ops[i] = _lib.MulMatOp(wt.data_ptr(), xd[m].data_ptr(), y.data_ptr(), m, n, k, 1 if i in (1, 4, 6) else 0, 0)
         want.append(oracle.gemm(w, oracle.quantize_rows(xs[m]), m, n, k, threads=4))
-    need = q8._lib.lib().nh_q8_0_mul_mat_workspace_bytes(8, k)
+    need = q8._lib.lib().nh_q8_0_mul_mat_workspace_bytes(24, k)
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    assert [q8.plan_mul_mat(m, n, k)["quantize_launch"] for m, n in shapes] == [False] * 5 + [True] * 2
     _lib.check("nh_q8_0_mul_mat_batch", q8._lib.lib().nh_q8_0_mul_mat_batch(ops, len(shapes), ws.data_ptr(), need, torch.cuda.current_stream().cuda_stream))
     for i in range(len(shapes)):
         assert rel_l2(to_host(keep[2 * i + 1]), want[i]) <= REL_L2_TOL, i
