@@ -66,6 +66,7 @@ template<int CTRL> __device__ __forceinline__ float lane_pattern(float x) {
 }
 constexpr int DPP_QUAD_SWAP_1	 = 0xB1; // quad_perm [1, 0, 3, 2]: lane ^ 1
 constexpr int DPP_QUAD_SWAP_2	 = 0x4E; // quad_perm [2, 3, 0, 1]: lane ^ 2
+constexpr int DPP_ROW_ROTATE_8	 = 0x128; // row_ror:8: lane (i + 8) % 16 of the same 16-lane row, i.e. lane ^ 8
 constexpr int DPP_ROW_HALF_MIRROR = 0x141; // lane i <-> 7 - i within each group of eight: pairs the two quads of the group
 
 // One lane's share of quantize_row_q8_0 (reference cpu/avx_2.hpp:4439-4489): eight consecutive lanes (a group aligned to eight)
@@ -157,11 +158,15 @@ __device__ __forceinline__ float sumsq_fold(float p, float4 v) {
 	p = fmaf(v.z, v.z, p);
 	return fmaf(v.w, v.w, p);
 }
+// (distances 8, 2 and 1 by lane patterns -- a rotation of a 16-lane row by 8 and the two quad swaps reach exactly lane ^ 8, ^ 2, ^ 1 --
+// the others through the LDS crossbar: same partners, same sums)
 __device__ __forceinline__ float wave_sum_butterfly(float p) {
-#pragma unroll
-	for (int off = 32; off >= 1; off >>= 1) {
-		p = __fadd_rn(p, __shfl_xor(p, off));
-	}
+	p = __fadd_rn(p, __shfl_xor(p, 32));
+	p = __fadd_rn(p, __shfl_xor(p, 16));
+	p = __fadd_rn(p, lane_pattern<DPP_ROW_ROTATE_8>(p));
+	p = __fadd_rn(p, __shfl_xor(p, 4));
+	p = __fadd_rn(p, lane_pattern<DPP_QUAD_SWAP_2>(p));
+	p = __fadd_rn(p, lane_pattern<DPP_QUAD_SWAP_1>(p));
 	return p;
 }
 // lane's share of run `wave` of a row of `groups` 128-value groups (K % 128 == 0)
