@@ -278,7 +278,7 @@ def main() -> int:
         torch.cuda.empty_cache()
         # the third named kernel (stand-alone activation quantize) and the two other benchmark configurations, compact
         qz = side_workload("quantize", 100, 10)
-        result["quantize"] = {"config": qz["config"], "roofline": qz["roofline"], "fused_forms": qz["fused_forms"]}
+        result["quantize"] = {"config": qz["config"], "roofline": qz["roofline"], "fused_forms": qz["fused_forms"], "streaming": qz["streaming"]}
         cross = side_workload("crossover", 100, 10)
         result["crossover"] = {"workload": cross["config"]["workload"], "unit": "us per nh_q8_0_mul_mat call (activation quantize included)",
                                "rows": [{k: r[k] for k in ("M", "N", "K", "us", "kernel", "pct_hbm", "pct_mfma")} for r in cross["rows"]]}
@@ -504,12 +504,35 @@ def side_workload(kind: str, steps: int, warmup: int) -> dict:
         for entry, f, b in (("nh_q8_0_rms_norm_quantize_tiled", fn_norm, nbytes + 4 * K), ("nh_q8_0_silu_mul_quantize_tiled", fn_silu, nbytes + 4 * M * K)):
             _, ks, _ = timed(0, f, 1)
             fused.append({"entry": entry, "avg_launch_us": round(ks * 1e6, 3), "bytes_per_launch": b, "GBs": round(b / ks / 1e9, 1)})
+        # the same three entry points at a size that streams from HBM (a long prompt: 8192 rows, inputs rotated over two buffers)
+        del up
+        Ml = 8192
+        xl = [q8_0.fill_activations(10 + i, Ml * K).reshape(Ml, K) for i in range(2)]
+        ul = q8_0.fill_activations(12, Ml * K).reshape(Ml, K)
+        outl = torch.empty(q8_0.tiled_bytes(Ml, K), dtype=torch.uint8, device=x.device)
+        nbl = 4 * Ml * K + Ml * (K // 32) * 34
+        turn = [0]
+
+        def pick():
+            turn[0] ^= 1
+            return xl[turn[0]]
+
+        streaming = []
+        for entry, f, b in (
+            ("nh_q8_0_quantize_tiled", lambda: _lib.check("q", lib.nh_q8_0_quantize_tiled(pick().data_ptr(), outl.data_ptr(), Ml, K, stream)), nbl),
+            ("nh_q8_0_rms_norm_quantize_tiled", lambda: _lib.check("q", lib.nh_q8_0_rms_norm_quantize_tiled(pick().data_ptr(), nw.data_ptr(), C.c_float(1e-5), outl.data_ptr(), Ml, K, stream)), nbl + 4 * K),
+            ("nh_q8_0_silu_mul_quantize_tiled", lambda: _lib.check("q", lib.nh_q8_0_silu_mul_quantize_tiled(pick().data_ptr(), ul.data_ptr(), outl.data_ptr(), Ml, K, stream)), nbl + 4 * Ml * K),
+        ):
+            _, ks, _ = timed(0, f, 1)
+            streaming.append({"entry": entry, "rows": Ml, "avg_launch_us": round(ks * 1e6, 2), "bytes_per_launch": b, "GBs": round(b / ks / 1e9, 1), "frac_of_hbm_peak": round(b / ks / 1e9 / HBM_PEAK_GBS, 4)})
+        del xl, ul, outl
         return {
             "fused_forms": fused,
+            "streaming": streaming,
             "metric": "Q8_0 activation quantize GB/s", "value": round(nbytes / wall / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
             "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "dtype": "fp32 -> int8 + fp16 scale", "data": "synthetic",
             "config": {"workload": f"activation quantize, fp32 [{M}x{K}] -> tiled Q8_0 (cache-resident at this size: 10.6 MB)"},
-            "roofline": {"bound": "hbm", "kernel": "nh::quantize_kernel<true>", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "roofline": {"bound": "hbm", "kernel": "nh::quantize_kernel<TILED=true, SILU_MUL=false, PASSES=1>", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": round(ksec * 1e6, 3), "launches_timed": n},
         }
 

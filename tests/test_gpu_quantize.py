@@ -69,6 +69,20 @@ def test_quantize_tiled_matches_blocks(q8, oracle):
             assert not full[m:].any()
 
 
+@pytest.mark.parametrize("m,k", [(1030, 4096), (8200, 512), (2048, 8192)])
+def test_quantize_two_blocks_per_thread(q8, oracle, m, k):
+    # from 2^20 float4s on a thread takes two, a grid's worth of threads apart: same bytes, both layouts, ragged last strip included
+    rng = np.random.default_rng(m + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[m // 2] = 0.0
+    want = oracle.quantize_rows(x)
+    assert np.array_equal(to_host(q8.quantize_row_q8_0(to_dev(x))), want)
+    tiled = q8.quantize_row_q8_0(to_dev(x), tiled=True)
+    rows = (m + 31) // 32 * 32
+    full = to_host(q8.untile(tiled, rows, k)).reshape(rows, -1)
+    assert np.array_equal(full[:m], want) and not full[m:].any()
+
+
 def test_quantize_empty_and_errors(q8):
     import torch
 

@@ -26,6 +26,21 @@ def test_rms_norm_quantize_bit_exact(q8, oracle, m, k):
     assert np.array_equal(to_host(q8.untile(tiled, m, k)).reshape(m, -1), want)
 
 
+@pytest.mark.parametrize("m,k", [(2048, 4096), (2050, 1664), (2048, 8192), (2100, 128), (2049, 2048), (4096, 640)])
+def test_rms_norm_quantize_eight_rows_per_workgroup(q8, oracle, m, k):
+    # From 2048 rows on the tiled form takes eight rows per workgroup (whole 128-byte lines of the operand tiles per store, the
+    # rows read once): one and two float4s per lane and run, runs of unequal length (13 and 5 groups over 16 runs), a single
+    # group, a ragged last strip whose padding rows must come out as zero blocks.  Same bytes as the CPU checker.
+    x, w = row_inputs(m + k, m, k)
+    x[7] = 0.0
+    want = oracle.rms_norm_quantize_rows(x, w, EPS)
+    tiled = q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS, tiled=True)
+    rows = (m + 31) // 32 * 32
+    full = to_host(q8.untile(tiled, rows, k)).reshape(rows, -1)
+    assert np.array_equal(full[:m], want)
+    assert not full[m:].any()
+
+
 @pytest.mark.parametrize("k", [128, 1024, 4096, 8192, 14336])
 def test_norm_inside_the_mat_vec_stages_the_same_bytes(q8, oracle, k):
     # K <= 8192: the in-chunk reduction (weights already in flight); 14336: the up-front form
