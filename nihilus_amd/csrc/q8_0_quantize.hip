@@ -145,15 +145,15 @@ __global__ __launch_bounds__(1024) void rms_norm_quantize_kernel(const float* __
 // consecutive rows own whole lines.  Waves 2r and 2r + 1 take row r: runs 8 (w % 2) .. + 7 of the fixed-order sum of squares,
 // each lane the float4s that the 16-wave form gives lane `lane` of wave `run` -- the same per-lane sums, butterflies and order
 // of the sixteen run sums, hence the same scale and the same bytes -- kept in registers for the quantizer, so the rows are read
-// once.  The quants and scales go to an LDS image of the eight rows' share of the tiles ([group][tile][half][row][16 bytes], then
+// once (non-temporal loads of the rows measured no different: the launch is bound by its stores).  The quants and scales go to an LDS image of the eight rows' share of the tiles ([group][tile][half][row][16 bytes], then
 // [group][row][4 scales]) and from there to memory as whole lines, 16 bytes per lane.  F4: float4s per lane and run.
 template<int F4>
-__global__ __launch_bounds__(1024) void rms_norm_quantize_rows8_kernel(const float* __restrict__ x, const float* __restrict__ norm_w, float eps, uint8_t* __restrict__ out, int64_t M, int K) {
+__global__ __launch_bounds__(1024, F4 == 1 ? 8 : 4) void rms_norm_quantize_rows8_kernel(const float* __restrict__ x, const float* __restrict__ norm_w, float eps, uint8_t* __restrict__ out, int64_t M, int K) {
 	__shared__ __align__(16) uint8_t image[F4 * 4096 * 8 + F4 * 32 * 64]; // K * 8 bytes of quants, then K / 128 * 64 bytes of scales (K <= 4096 F4)
 	__shared__ float red[8][16];
 	const int tid	 = threadIdx.x;
 	const int lane	 = tid & 63;
-	const int wave	 = tid >> 6;
+	const int wave	 = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: the runs' bounds stay in scalar registers
 	const int row8	 = wave >> 1; // which of the workgroup's eight rows
 	const int64_t m0 = static_cast<int64_t>(blockIdx.x) * 8;
 	const int64_t m	 = m0 + row8;
