@@ -283,9 +283,13 @@ template<int CHUNKS> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_l
 			return;
 		}
 		// ---- a (32-row strip, K split) of the down projection against the published activation, + ffn_inp ----
-		const int splits = 1 << a.split_shift;
-		const int gstrip = c >> a.split_shift;
-		const int split	 = c & (splits - 1);
+		// (K part first, strip second: the first K part's activation blocks come from the first gate/up workgroups, so the down
+		// workgroups that are dispatched first can finish instead of holding their CUs until the last gate/up workgroup is done:
+		// a LLaMA-3-70B block 150.2 -> 145.5 us; no difference at the LLaMA-3-8B shapes, two K parts)
+		const int splits   = 1 << a.split_shift;
+		const int strips_d = (a.n_embd + STRIP_ROWS - 1) / STRIP_ROWS;
+		const int split	   = c / strips_d;
+		const int gstrip   = c - split * strips_d;
 		int g0, g1;
 		wave_k_range(a.groups_f, a.split_shift, split, GEMV_WAVES, wave, g0, g1);
 		const uint8_t* w_strip = a.w_down + macro_offset(gstrip, 0, a.groups_f);
