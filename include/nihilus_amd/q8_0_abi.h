@@ -97,6 +97,15 @@ int nh_q8_0_last_error(void);
 /* Resets that error and returns what it held (NH_OK or NH_ERR_DEVICE_TIMEOUT): for the owner of the failed launch, once it has
  * dealt with the NaN output.  A sync of an unrelated stream never resets it. */
 int nh_q8_0_clear_error(void);
+/* Whether a launch may contain workgroups that wait (for a bounded time) for other workgroups of the same launch: the decode FFN
+ * as one launch, a block's mat-vecs as one launch, the normalised row that the first workgroups of a large mat-vec work out for the
+ * rest.  Those forms rest on workgroups being dispatched in index order, which holds on this hardware and is nowhere promised.
+ * enabled = 0 switches them off for the whole process: nh_q8_0_ffn_f32 and nh_q8_0_decode_layer_f32 then run as the launches they
+ * stand for (what a capturing stream gets), each depending on the one before only through stream order -- the reference's own
+ * model, one kernel per op back to back (cuda/thread_pool.hpp:46-67) -- and every workgroup of a mat-vec with a norm works the
+ * row out itself.  Same results (the fp32 sums of the one-launch forms may be cut differently: 1e-6 relative).  Returns the
+ * previous setting (1 or 0); 1 by default.  Takes effect for calls made afterwards; needs no GPU. */
+int nh_q8_0_set_in_kernel_waits(int enabled);
 /* Allocates, for the current device, the two internal scratch buffers that K-split launches hand partial sums through
  * (about 2.6 MiB and 16 MiB; otherwise made by the first launch that needs one).  After it no launch entry point of this library
  * allocates device memory: call it once per device before capturing launches into a HIP graph or entering a serving loop.

@@ -53,6 +53,7 @@ SIGNATURES = {
     "nh_q8_0_last_error": (_int, []),
     "nh_q8_0_clear_error": (_int, []),
     "nh_q8_0_debug_set_spin_limit": (_int, [_i64]),
+    "nh_q8_0_set_in_kernel_waits": (_int, [_int]),
     "nh_q8_0_debug_plan_mul_mat": (_int, [_i64, _i64, _i64, _vp]),
     "nh_q8_0_gemv_tiled_residual_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "nh_q8_0_gemv_tiled_multi_f32": (_int, [C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64), _i64, _vp, _i64, _vp]),

@@ -203,6 +203,10 @@ int nh_q8_0_clear_error(void) {
 	return nh::read_device_error(true) != nh::DEVICE_ERROR_NONE ? NH_ERR_DEVICE_TIMEOUT : NH_OK;
 }
 
+int nh_q8_0_set_in_kernel_waits(int enabled) {
+	return nh::set_in_kernel_waits(enabled != 0) ? 1 : 0;
+}
+
 int nh_q8_0_debug_set_spin_limit(int64_t polls) {
 	// a test hook in a production library: it only works for a process that asked for it
 	const char* hooks = std::getenv("NH_Q8_0_DEBUG_HOOKS");

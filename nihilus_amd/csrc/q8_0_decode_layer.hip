@@ -402,7 +402,7 @@ hipError_t launch_decode_layer(const void* w_o, const float* attn, const float* 
 	for (int i = 0; i < count_next; ++i) {
 		next_strips += (n_next[i] + STRIP_ROWS - 1) / STRIP_ROWS;
 	}
-	if (!decode_layer_chains(n_embd, n_ff, next_strips) || stream_is_capturing(s)) {
+	if (!decode_layer_chains(n_embd, n_ff, next_strips) || stream_is_capturing(s) || !in_kernel_waits_enabled()) {
 		// the same three steps as launches of their own
 		const void* w1[1]  = { w_o };
 		float* y1[1]	   = { ffn_inp };

@@ -235,7 +235,8 @@ hipError_t launch_ffn_decode(const void* w_gate, const void* w_up, const void* w
 	if (e != hipSuccess) {
 		return e;
 	}
-	if (stream_is_capturing(s)) {
+	if (stream_is_capturing(s) || !in_kernel_waits_enabled()) {
+		// (Also what a caller gets who has switched waits between the workgroups of a launch off.)
 		// A replayed graph runs the kernel with the epoch it was captured with, so the published blocks of one replay would
 		// pass for those of the next.  Under capture the step is three launches instead, none of which keeps state between
 		// launches: gate/up mat-vecs (norm inside) -> SiLU * up -> quantize -> down mat-vec (+ residual).  The gate / up

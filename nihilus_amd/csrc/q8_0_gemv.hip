@@ -13,6 +13,7 @@
 // reduction; halves and waves are combined once through LDS in a fixed order (run-to-run bit-stable).
 #include "q8_0_plan.h"
 
+#include <atomic>
 #include <mutex>
 
 namespace nh {
@@ -319,6 +320,16 @@ unsigned read_device_error(bool clear) {
 	return clear ? __atomic_exchange_n(word, static_cast<unsigned>(DEVICE_ERROR_NONE), __ATOMIC_RELAXED) : __atomic_load_n(word, __ATOMIC_RELAXED);
 }
 
+namespace {
+	std::atomic<bool> in_kernel_waits{ true };
+}
+bool in_kernel_waits_enabled() {
+	return in_kernel_waits.load(std::memory_order_relaxed);
+}
+bool set_in_kernel_waits(bool enabled) {
+	return in_kernel_waits.exchange(enabled, std::memory_order_relaxed);
+}
+
 void set_published_spin_limit(int limit) {
 	std::lock_guard<std::mutex> g(scratch_lock);
 	published_spin_limit = limit < 1 ? 1 : (limit > PUBLISHED_SPIN_LIMIT ? PUBLISHED_SPIN_LIMIT : limit);
@@ -483,7 +494,7 @@ static hipError_t launch_gemv_tiled_any(const void* const* W, float* const* y, c
 		p.tiles	 = (p.groups + GEMV_WAVES - 1) / GEMV_WAVES;
 	}
 	gemv_scratch sc;
-	if (p.splits == 1 && norm_w && x_is_f32 && dump_mode == DUMP_NONE && !noalloc && gemv_shares_x(p, 1) && !stream_is_capturing(s)) {
+	if (p.splits == 1 && norm_w && x_is_f32 && dump_mode == DUMP_NONE && !noalloc && gemv_shares_x(p, 1) && !stream_is_capturing(s) && in_kernel_waits_enabled()) {
 		// the normalised, quantized row goes from the first strip's workgroups to the others through the scratch, tagged with a
 		// fresh epoch; not under capture, where a replay could not renew the epoch: there every workgroup works the row out
 		const hipError_t e = get_gemv_scratch(&sc, true, s);

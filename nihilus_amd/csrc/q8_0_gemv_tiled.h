@@ -481,6 +481,11 @@ hipError_t get_gemv_scratch(gemv_scratch* out, bool next_epoch = false, hipStrea
 // Reads the current device's error word (DEVICE_ERROR_NONE if no scratch exists yet); clear = true also resets it.
 unsigned read_device_error(bool clear);
 void set_published_spin_limit(int limit);
+// Whether launches may contain workgroups that wait for other workgroups of the same launch (the one-launch FFN, the chained block,
+// the norm row shared between the workgroups of a large mat-vec).  On by default; off, those calls take the forms a capturing
+// stream gets: several launches, or every workgroup working the row out itself.  Process-wide.
+bool in_kernel_waits_enabled();
+bool set_in_kernel_waits(bool enabled); // returns the previous setting
 
 // How a tiled mat-vec launch is cut: `splits` workgroups per strip, each of 16 waves owning <= `tiles` groups.
 struct gemv_plan {
