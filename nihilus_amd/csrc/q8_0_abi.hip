@@ -668,7 +668,7 @@ static int mul_mat_common(const void* W_tiled, const float* x, const float* resi
 	if (M == 1) { // quantize fused into the mat-vec: the workspace stays unused
 		return residual ? nh_q8_0_gemv_tiled_residual_f32(W_tiled, x, residual, y, N, K, stream) : nh_q8_0_gemv_tiled_f32(W_tiled, x, y, N, K, stream);
 	}
-	if (plan.kernel == nh::MM_GEMV_ROWS_MFMA) { // up to eight rows: the streaming kernel with the rows as an MFMA operand
+	if (plan.kernel == nh::MM_GEMV_ROWS_MFMA) { // four to sixteen rows on small matrices: the streaming kernel with the rows as an MFMA operand
 		NH_REQUIRE(W_tiled && y, NH_ERR_NULL_POINTER);
 		NH_REQUIRE(aligned16(W_tiled) && aligned16(y) && aligned16(residual), NH_ERR_ALIGNMENT);
 		NH_TRY(require_device());

@@ -84,7 +84,7 @@ inline gemm_skinny_cut plan_gemm_skinny(int64_t M, int64_t N, int64_t K) {
 	return c;
 }
 
-// A mat-mat on tiled, already quantized operands (nh_q8_0_gemm_tiled and the second half of nh_q8_0_mul_mat for M > 5).
+// A mat-mat on tiled, already quantized operands (nh_q8_0_gemm_tiled, and the second half of nh_q8_0_mul_mat wherever the activations are quantized by a launch of their own).
 struct gemm_plan {
 	int kernel; // MM_GEMM_SKINNY, MM_GEMM_TILE_STREAM or MM_GEMM_TILE (MM_NOTHING for an empty problem)
 	gemm_tile_cut tile; // when a tile kernel runs
