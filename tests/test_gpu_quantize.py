@@ -83,6 +83,18 @@ def test_quantize_two_blocks_per_thread(q8, oracle, m, k):
     assert np.array_equal(full[:m], want) and not full[m:].any()
 
 
+def test_quantize_either_side_of_the_size_where_a_thread_takes_two_blocks(q8, oracle):
+    # 2^20 float4s = 2^17 blocks: shapes just below, at and above it, odd row counts, both layouts
+    for m, k in [(1023, 4096), (1024, 4096), (1025, 4096), (4097, 1024), (257, 16384)]:
+        rng = np.random.default_rng(m + k)
+        x = (rng.standard_normal((m, k)) * rng.uniform(0.01, 100.0)).astype(np.float32)
+        want = oracle.quantize_rows(x)
+        assert np.array_equal(to_host(q8.quantize_row_q8_0(to_dev(x))), want), (m, k)
+        rows = (m + 31) // 32 * 32
+        full = to_host(q8.untile(q8.quantize_row_q8_0(to_dev(x), tiled=True), rows, k)).reshape(rows, -1)
+        assert np.array_equal(full[:m], want) and not full[m:].any(), (m, k)
+
+
 def test_quantize_empty_and_errors(q8):
     import torch
 

@@ -41,6 +41,20 @@ def test_rms_norm_quantize_eight_rows_per_workgroup(q8, oracle, m, k):
     assert not full[m:].any()
 
 
+def test_rms_norm_quantize_either_side_of_the_row_count_where_the_form_changes(q8, oracle):
+    # seeded random shapes around 2048 rows (one row per workgroup below, eight from there on) and K up to 8192 and beyond (the
+    # eight-row form stops at 8192): both forms and the hand-over between them give the checker's bytes
+    rng = np.random.default_rng(2048)
+    shapes = [(2047, 384), (2048, 384), (2049, 384)] + [(int(rng.integers(1990, 2120)), 128 * int(rng.integers(1, 65))) for _ in range(5)] + [(2050, 8320)]
+    for m, k in shapes:
+        x, w = row_inputs(m * 7 + k, m, k, scale=float(rng.uniform(0.1, 30.0)))
+        want = oracle.rms_norm_quantize_rows(x, w, EPS)
+        rows = (m + 31) // 32 * 32
+        full = to_host(q8.untile(q8.rms_norm_quantize(to_dev(x), to_dev(w), EPS, tiled=True), rows, k)).reshape(rows, -1)
+        assert np.array_equal(full[:m], want), (m, k)
+        assert not full[m:].any(), (m, k)
+
+
 @pytest.mark.parametrize("k", [128, 1024, 4096, 8192, 14336])
 def test_norm_inside_the_mat_vec_stages_the_same_bytes(q8, oracle, k):
     # K <= 8192: the in-chunk reduction (weights already in flight); 14336: the up-front form
