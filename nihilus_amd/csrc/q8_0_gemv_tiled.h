@@ -207,8 +207,21 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 			if (__builtin_amdgcn_ballot_w64(!fresh) == 0) {
 				break;
 			}
-			if (++spins >= spin_limit) {
-				timed_out = true;
+			// Not there yet: watch ONE word of the slice (its last; the same address in every lane, one request per poll) until it is
+			// this launch's, then read the whole slice again.  A wave that waits long -- a workgroup that became resident well before
+			// its producers are done -- polls 8 bytes at a time instead of the slice's 72 per block.
+			for (;;) {
+				if (++spins >= spin_limit) {
+					timed_out = true;
+					break;
+				}
+				__builtin_amdgcn_s_sleep(8);
+				const uint64_t last = __hip_atomic_load(pw + (n_words - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				if (static_cast<unsigned>(last >> 32) == epoch) {
+					break;
+				}
+			}
+			if (timed_out) {
 				// tell the host (an ordinary vector store to pinned host memory).  Done here, not where the NaN is set: kept for
 				// the end of the function the pointer and the branch cost the hot path 25 registers
 				if (lane == 0 && dump) {
@@ -216,7 +229,6 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 				}
 				break;
 			}
-			__builtin_amdgcn_s_sleep(8);
 		}
 #pragma unroll
 		for (int i = 0; i < PW_LOADS; ++i) {
