@@ -210,7 +210,7 @@ template<int CHUNKS> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_l
 		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
 		float acc = 0.0f, acc_up = 0.0f;
 		if constexpr (CHUNKS == 1) {
-			acc = gemv_chunk<2, X_PUBLISHED_EARLY, DUMP_NONE, false, 1, 2>(w_strip, a.x_words, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_e, lane, row_l, a.n_ff, false, a.epoch, nullptr, 0,
+			acc = gemv_chunk<2, X_PUBLISHED_EARLY_WATCH, DUMP_NONE, false, 1, 2>(w_strip, a.x_words, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_e, lane, row_l, a.n_ff, false, a.epoch, nullptr, 0,
 				a.spin_limit, w_other, &acc_up);
 		} else {
 			for (int gc = g0; gc < g1; gc += 2) {
@@ -360,7 +360,7 @@ template<int CHUNKS> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_l
 		wave_k_range(a.groups_e, 0, 0, GEMV_WAVES, wave, g0, g1);
 		const uint8_t* w_strip = a.next.W[sidx] + macro_offset(strip, 0, a.groups_e);
 		const int row_l		   = strip * STRIP_ROWS + (lane & 31);
-		const float acc = gemv_chunk<CHAIN_TILES, X_PUBLISHED_EARLY, DUMP_NONE>(w_strip, a.x_words_next, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_e, lane, row_l, N, false, a.epoch, nullptr, 0,
+		const float acc = gemv_chunk<CHAIN_TILES, CHUNKS == 1 ? X_PUBLISHED_EARLY_WATCH : X_PUBLISHED_EARLY, DUMP_NONE>(w_strip, a.x_words_next, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_e, lane, row_l, N, false, a.epoch, nullptr, 0,
 			a.spin_limit);
 		red[wave][lane] = acc;
 		__syncthreads();

@@ -103,7 +103,7 @@ template<int TILES, bool LOOP, bool NORM, bool PAIR = false> __global__ __launch
 				norm_state.epoch   = a.epoch;
 				acc				   = walk.template operator()<X_F32, true>(a.x, nullptr, &norm_state);
 			} else {
-				acc = walk.template operator()<X_PUBLISHED_EARLY, false>(a.x_words, a.error_word, nullptr);
+				acc = walk.template operator()<X_PUBLISHED_EARLY_WATCH, false>(a.x_words, a.error_word, nullptr);
 			}
 		} else if constexpr (PAIR) {
 			acc = walk.template operator()<X_F32, false>(a.x, nullptr, nullptr);

@@ -170,7 +170,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_tiled_kernel(gemv_segmen
 			norm_state.epoch   = epoch;
 			acc				   = walk.template operator()<XF32 ? X_F32 : X_BLOCKS, true>(xin, dump, &norm_state);
 		} else if constexpr (DUMP == DUMP_NONE) {
-			acc = walk.template operator()<X_PUBLISHED_EARLY, false>(x_words, error_word, nullptr);
+			acc = walk.template operator()<X_PUBLISHED_EARLY_WATCH, false>(x_words, error_word, nullptr);
 		}
 	} else if constexpr (!LOOP) {
 		acc = gemv_chunk<TILES, XF32, DUMP, false, RS>(w_strip, xin, dump, xs_q[wave], xs_d[wave], g0, g1 - g0, groups, lane, row_l, N, gstrip == 0, 0, nullptr, rowpart);

@@ -30,10 +30,13 @@ enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
 //               wait is bounded: after `spin_limit` polls the wave gives up, returns NaN and stores a non-zero code
 //               in the device-visible error word that `dump` names in this mode (host memory that the next
 //               nh_stream_sync / nh_q8_0_last_error reads), so the kernel always drains and the failure reaches the host.
+//   X_PUBLISHED_EARLY_WATCH  X_PUBLISHED_EARLY for waves that may wait long for a row that ONE workgroup publishes: after two polls of the
+//               whole slice a waiting wave watches a single word of it until that carries the epoch (8 bytes per poll instead of 72 per block)
 //   X_PUBLISHED_EARLY  the same, with a first read of the words ahead of the weight loads: for slices that are usually there
 //               already when the workgroup starts (a launch's input row, published by its first workgroups).
-enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2, X_PUBLISHED_EARLY = 3 };
+enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2, X_PUBLISHED_EARLY = 3, X_PUBLISHED_EARLY_WATCH = 4 };
 constexpr int PUBLISHED_SPIN_LIMIT = 1 << 20;
+constexpr int PUBLISHED_FULL_POLLS = 2; // polls of a whole slice before a waiting wave starts watching one word of it
 constexpr int PUBLISHED_WORDS	   = 9; // per block: quant dwords 0..7, then the scale
 // codes a kernel leaves in the device-visible error word (nh_q8_0_last_error reports them as NH_ERR_DEVICE_TIMEOUT)
 enum device_error : unsigned { DEVICE_ERROR_NONE = 0, DEVICE_ERROR_PUBLISH_TIMEOUT = 1 };
@@ -90,8 +93,9 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	static_assert(MATS == 1 || (MATS == 2 && RS == 1 && DUMP == DUMP_NONE), "two matrices: whole strips, production form");
 	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
-	constexpr bool XPUB = XMODE == X_PUBLISHED || XMODE == X_PUBLISHED_EARLY; // the slice is read as tagged words
-	constexpr bool EARLY = XMODE == X_PUBLISHED_EARLY; // ... with a first look before the weight loads go out
+	constexpr bool WATCH = XMODE == X_PUBLISHED_EARLY_WATCH;
+	constexpr bool EARLY = XMODE == X_PUBLISHED_EARLY || WATCH; // ... with a first look before the weight loads go out
+	constexpr bool XPUB = XMODE == X_PUBLISHED || EARLY; // the slice is read as tagged words
 	static_assert(RS == 1 || RS == 2 || RS == 4, "a strip splits into 1, 2 or 4 row parts");
 	static_assert(RS == 1 || DUMP == DUMP_NONE, "the inspection variants run on whole strips");
 	constexpr int PART_ROWS = STRIP_ROWS / RS; // rows this workgroup owns
@@ -190,6 +194,7 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	if constexpr (XPUB) {
 		int spins	= 0;
 		bool looked = EARLY; // the first set of words is already on its way
+		bool watched = !WATCH; // the slice's last word has been seen to be this launch's
 		for (;;) {
 			if (!looked) {
 #pragma unroll
@@ -209,16 +214,21 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 			}
 			// Not there yet: watch ONE word of the slice (its last; the same address in every lane, one request per poll) until it is
 			// this launch's, then read the whole slice again.  A wave that waits long -- a workgroup that became resident well before
-			// its producers are done -- polls 8 bytes at a time instead of the slice's 72 per block.
-			for (;;) {
-				if (++spins >= spin_limit) {
-					timed_out = true;
-					break;
-				}
-				__builtin_amdgcn_s_sleep(8);
+			// its producers are done -- polls 8 bytes at a time instead of the slice's 72 per block.  Once that word has come the
+			// rest is polled as a whole (a slice with several producers: watching one word first would put a second round trip
+			// into every further poll).
+			if (++spins >= spin_limit) {
+				timed_out = true;
+			}
+			__builtin_amdgcn_s_sleep(8);
+			while (!watched && !timed_out && spins > PUBLISHED_FULL_POLLS) {
 				const uint64_t last = __hip_atomic_load(pw + (n_words - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 				if (static_cast<unsigned>(last >> 32) == epoch) {
-					break;
+					watched = true;
+				} else if (++spins >= spin_limit) {
+					timed_out = true;
+				} else {
+					__builtin_amdgcn_s_sleep(8);
 				}
 			}
 			if (timed_out) {
