@@ -258,7 +258,7 @@ template<int CHUNKS> __global__ __launch_bounds__(GEMV_WAVES * 64) void decode_l
 			wave_k_range(a.groups_f, 0, 0, GEMV_WAVES, wave, g0, g1);
 			const uint8_t* w_strip = a.w_down + macro_offset(gstrip, 0, a.groups_f);
 			const int row_l		   = gstrip * STRIP_ROWS + (lane & 31);
-			const float acc = gemv_chunk<CHAIN_DOWN_ROWS_TILES, X_PUBLISHED, DUMP_NONE, false, 2>(w_strip, a.act_words, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_f, lane, row_l, a.n_embd, false,
+			const float acc = gemv_chunk<CHAIN_DOWN_ROWS_TILES, X_PUBLISHED_WATCH, DUMP_NONE, false, 2>(w_strip, a.act_words, a.error_word, xs_q[wave], xs_d[wave], g0, g1 - g0, a.groups_f, lane, row_l, a.n_embd, false,
 				a.epoch, nullptr, rowpart, a.spin_limit);
 			red[wave][lane] = acc;
 			__syncthreads();

@@ -32,9 +32,10 @@ enum gemv_dump : int { DUMP_NONE = 0, DUMP_SUMS = 1, DUMP_X = 2 };
 //               nh_stream_sync / nh_q8_0_last_error reads), so the kernel always drains and the failure reaches the host.
 //   X_PUBLISHED_EARLY_WATCH  X_PUBLISHED_EARLY for waves that may wait long for a row that ONE workgroup publishes: after two polls of the
 //               whole slice a waiting wave watches a single word of it until that carries the epoch (8 bytes per poll instead of 72 per block)
+//   X_PUBLISHED_WATCH  X_PUBLISHED with the same watching (a slice of several producers whose last block is the last to come)
 //   X_PUBLISHED_EARLY  the same, with a first read of the words ahead of the weight loads: for slices that are usually there
 //               already when the workgroup starts (a launch's input row, published by its first workgroups).
-enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2, X_PUBLISHED_EARLY = 3, X_PUBLISHED_EARLY_WATCH = 4 };
+enum gemv_xmode : int { X_BLOCKS = 0, X_F32 = 1, X_PUBLISHED = 2, X_PUBLISHED_EARLY = 3, X_PUBLISHED_EARLY_WATCH = 4, X_PUBLISHED_WATCH = 5 };
 constexpr int PUBLISHED_SPIN_LIMIT = 1 << 20;
 constexpr int PUBLISHED_FULL_POLLS = 2; // polls of a whole slice before a waiting wave starts watching one word of it
 constexpr int PUBLISHED_WORDS	   = 9; // per block: quant dwords 0..7, then the scale
@@ -93,9 +94,9 @@ __device__ __forceinline__ float gemv_chunk_n(const uint8_t* __restrict__ w_stri
 	static_assert(MATS == 1 || (MATS == 2 && RS == 1 && DUMP == DUMP_NONE), "two matrices: whole strips, production form");
 	constexpr int cnt	= CNT;
 	constexpr bool XF32 = XMODE == X_F32; // the slice is quantized here, from fp32
-	constexpr bool WATCH = XMODE == X_PUBLISHED_EARLY_WATCH;
-	constexpr bool EARLY = XMODE == X_PUBLISHED_EARLY || WATCH; // ... with a first look before the weight loads go out
-	constexpr bool XPUB = XMODE == X_PUBLISHED || EARLY; // the slice is read as tagged words
+	constexpr bool WATCH = XMODE == X_PUBLISHED_EARLY_WATCH || XMODE == X_PUBLISHED_WATCH;
+	constexpr bool EARLY = XMODE == X_PUBLISHED_EARLY || XMODE == X_PUBLISHED_EARLY_WATCH; // ... with a first look before the weight loads go out
+	constexpr bool XPUB = XMODE == X_PUBLISHED || XMODE == X_PUBLISHED_WATCH || EARLY; // the slice is read as tagged words
 	static_assert(RS == 1 || RS == 2 || RS == 4, "a strip splits into 1, 2 or 4 row parts");
 	static_assert(RS == 1 || DUMP == DUMP_NONE, "the inspection variants run on whole strips");
 	constexpr int PART_ROWS = STRIP_ROWS / RS; // rows this workgroup owns
